@@ -50,12 +50,14 @@ def parse_config(c: Mapping[str, Any]) -> ModelConfig:
     """config.json (as a dict) -> ModelConfig.
 
     As model/Families.java:57-59, :95-106: ``model_type`` selects the entry; when it is missing it is
-    inferred from ``architectures[0]``; a declared architecture that does not belong to the model type
+    inferred from ``architectures[0]`` (or a single ``architecture`` string); a declared architecture that does not belong to the model type
     is refused with the list of what is supported.
     """
     if not isinstance(c, Mapping):
         raise ConfigError("config.json must hold a JSON object")
     archs = c.get("architectures")
+    if archs is None and isinstance(c.get("architecture"), str):  # a config that names its one design directly
+        archs = [c["architecture"]]
     declared = str(archs[0]) if isinstance(archs, (list, tuple)) and archs else None
     model_type = c.get("model_type")
     if not isinstance(model_type, str):

@@ -121,6 +121,54 @@ class GqaSpec:
         return self.heads // self.kv_heads
 
 
+@dataclass(frozen=True)
+class LatentAttentionNames:
+    """Tensor names of a latent-attention mixer under the layer's prefix (no ending: the tensors are named bare)."""
+
+    dq: str = "mix.dq"
+    dq_norm: str = "mix.dq.norm"
+    uq: str = "mix.uq"
+    dkv: str = "mix.dkv"
+    dkv_norm: str = "mix.dkv.norm"
+    uk: str = "mix.uk"
+    uv: str = "mix.uv"
+    sink: str = "mix.sink"
+    gate: str = "mix.g"
+    o: str = "mix.o"
+    ending: str = ""
+
+
+@dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Attention whose queries, keys and values pass through low-rank latents.
+
+    Per position the layer caches the RMS-normed latent c (``kv_rank`` numbers) and one rotated key part of
+    ``rot_dim`` numbers that all heads share; head h's unrotated key is W_uk[h] c and its value W_uv[h] c. A head's
+    query has ``dim`` unrotated and ``rot_dim`` rotated entries and comes from a normed latent of ``q_rank``.
+    ``window`` 0 = all earlier keys, else the query at p sees keys p + 1 - window .. p. ``sink``: a learned number
+    per head whose exponential joins the softmax's denominator. ``out_gate``: the concatenated heads are multiplied
+    by sigmoid(W_g h) before the output product. ``owns_cache`` False: the run reads the cache of an earlier run (the
+    schedule says which) and has no W_dkv. ``keep``: the window the cache must honour (the widest of the runs that
+    read it; 0 = everything), which is what the cache manager sees."""
+
+    heads: int
+    dim: int
+    rot_dim: int
+    vdim: int
+    q_rank: int
+    kv_rank: int
+    scale: float
+    eps: float
+    window: int = 0
+    keep: int = 0
+    position: Optional[int] = 0
+    sink: bool = True
+    out_gate: bool = True
+    owns_cache: bool = True
+    names: LatentAttentionNames = LatentAttentionNames()
+    kind: str = "latent_attention"
+
+
 # --------------------------------------------------------------------------- feed-forwards
 
 
@@ -133,16 +181,50 @@ class GatedMlpNames:
     up: str = "mlp.up_proj"
     down: str = "mlp.down_proj"
     gate_up: Optional[str] = None
+    ending: str = ".weight"  # what follows each name in the checkpoint ("" where tensors are named bare)
 
 
 @dataclass(frozen=True)
 class GatedMlpSpec:
-    """Dense gated feed-forward: down(act(gate x) * up x) (model/Mlp.java:7-22)."""
+    """Dense gated feed-forward: down(act(gate x) * up x) (model/Mlp.java:7-22). ``activation`` names the gate
+    function of the product kernels: "silu", "gelu_tanh", or "swish_clamped" (g = min(gate, limit), u = clamp(up,
+    -limit, limit), out = g * sigmoid(1.702 g) * (u + 1), with ``limit`` given here)."""
 
     hidden: int
     activation: str = "silu"
     names: GatedMlpNames = GatedMlpNames()
+    limit: float = 0.0
     kind: str = "gated_mlp"
+
+
+@dataclass(frozen=True)
+class TableMoeNames:
+    """Tensor names of a table-routed mixture of experts under the layer's prefix: expert e's tensors are
+    ``<expert>{e}.<gate|up|down>``, the routing table ``table``, the shared expert's ``<shared>.<gate|up|down>``."""
+
+    expert: str = "mlp.e"
+    gate: str = "gate"
+    up: str = "up"
+    down: str = "down"
+    table: str = "mlp.table"
+    shared: str = "mlp.shared"
+    ending: str = ""
+
+
+@dataclass(frozen=True)
+class TableMoeSpec:
+    """A mixture of small gated feed-forwards without a router: an integer table [vocab, top] gives every token id
+    its experts, each weighted 1 / top. Experts are "swish_clamped" gated feed-forwards of ``hidden`` with ``limit``;
+    ``shared`` (a GatedMlpSpec or None) runs for every token and is added."""
+
+    experts: int
+    top: int
+    hidden: int
+    limit: float
+    vocab: int
+    shared: Any = None
+    names: TableMoeNames = TableMoeNames()
+    kind: str = "table_moe"
 
 
 # --------------------------------------------------------------------------- layers and model
@@ -153,7 +235,7 @@ class LayerSpec:
     """One decoder layer: which mixer, which feed-forward, which norms, and how they are arranged.
 
     ``arrangement`` "prenorm": x += mixer(norm(x)); x += ffn(norm(x)) (model/LayerSpec.java:18-19,
-    cpu/CpuBackend.java:959-969). ``prefix`` is the tensor-name prefix of the layer's weights; the names under it
+    cpu/CpuBackend.java:959-969). ``ffn`` None: the layer has no feed-forward (and no second norm). ``prefix`` is the tensor-name prefix of the layer's weights; the names under it
     are data of the specs (here the two norms', in the mixer's and feed-forward's specs theirs), so a checkpoint
     that names or stacks its tensors differently is a matter of the parser.
     """
@@ -163,8 +245,9 @@ class LayerSpec:
     norm: Any
     prefix: str
     arrangement: str = "prenorm"
-    norm_in_name: str = "input_layernorm"  # under the prefix, without ``.weight``
+    norm_in_name: str = "input_layernorm"  # under the prefix, without the ending
     norm_post_name: str = "post_attention_layernorm"
+    name_ending: str = ".weight"
 
 
 @dataclass(frozen=True)

@@ -42,27 +42,54 @@ __device__ __forceinline__ float round_to<float>(float v) { return v; }
 template <>
 __device__ __forceinline__ float round_to<bf16_t>(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 
-// The gate function of the gated epilogue, out = gate(a . Wg) * (a . Wu), has a code that rides in bits 8 and up of an
-// entry point's `epilogue` argument (bits 0..7: 0 store, 1 add into fp32, 2 gated). One gate function is built:
-// code 0, SiLU, z / (1 + exp(-z)) (cpu/VectorKernels.java:637-639 of the reference). Every product kernel applies
-// gate_fn below and every entry point takes its argument apart with JLLM_TAKE_GATE, which refuses a code that is not
-// built with a message; another gate function is a case in gate_fn, a larger JLLM_GATE_COUNT, and the code handed
-// on to the kernels.
+// The gate function of the gated epilogue, out = gate(a . Wg, a . Wu), has a code that rides in bits 8 and up of an
+// entry point's `epilogue` argument (bits 0..7: 0 store, 1 add into fp32, 2 gated), and one parameter, `gate_limit`,
+// for the functions that have one. Built:
+//   0 silu           z / (1 + exp(-z)) * u   (cpu/VectorKernels.java:637-639 of the reference)
+//   1 gelu_tanh      0.5 z (1 + tanh(sqrt(2/pi) (z + 0.044715 z^3))) * u
+//   2 swish_clamped  g = min(z, limit), v = clamp(u, -limit, limit): g / (1 + exp(-1.702 g)) * (v + 1)
+// Every product kernel applies gated() below with the GateSpec its entry point made with JLLM_TAKE_GATE, which refuses a
+// code that is not built with a message; another gate function is a case in gated(), a larger JLLM_GATE_COUNT, and a
+// name in the Python face's table.
 #define JLLM_GATE_SILU 0
-#define JLLM_GATE_COUNT 1
-#define JLLM_TAKE_GATE(name, epilogue)                                                                       \
+#define JLLM_GATE_GELU_TANH 1
+#define JLLM_GATE_SWISH_CLAMPED 2
+#define JLLM_GATE_COUNT 3
+#define JLLM_SWISH_ALPHA 1.702f
+struct GateSpec {
+  int fn;
+  float limit;
+};
+#define JLLM_TAKE_GATE(name, epilogue, limit_, spec_)                                                        \
+  GateSpec spec_;                                                                                            \
   do {                                                                                                       \
     const int gate_ = (epilogue) >> 8;                                                                       \
     (epilogue) &= 0xff;                                                                                      \
     if (gate_ < 0 || gate_ >= JLLM_GATE_COUNT)                                                               \
-      JLLM_FAIL("%s: gate function %d of the gated epilogue is not built (0 = silu is)", name, gate_);        \
+      JLLM_FAIL("%s: gate function %d of the gated epilogue is not built (0 silu, 1 gelu_tanh, 2 swish_clamped are)", name, gate_); \
     if (gate_ != 0 && (epilogue) != 2) JLLM_FAIL("%s: a gate function without the gated epilogue", name);    \
+    if (gate_ == JLLM_GATE_SWISH_CLAMPED && !((limit_) > 0.f))                                               \
+      JLLM_FAIL("%s: the clamped gate needs a positive limit, got %g", name, (double)(limit_));              \
+    spec_.fn = gate_;                                                                                        \
+    spec_.limit = (limit_);                                                                                  \
   } while (0)
 // FAST: the hardware's exp2 and reciprocal (where the result is rounded to bf16 or added in fp32 anyway)
 template <bool FAST>
-__device__ __forceinline__ float gate_fn(float z) {
-  if (FAST) return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * z));
-  return z / (1.0f + expf(-z));
+__device__ __forceinline__ float sigmoid_times(float z, float slope) {  // z / (1 + exp(-slope z))
+  if (FAST) return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * slope * z));
+  return z / (1.0f + expf(-slope * z));
+}
+template <bool FAST>
+__device__ __forceinline__ float gated(float z, float u, GateSpec gs) {
+  if (gs.fn == JLLM_GATE_SILU) return sigmoid_times<FAST>(z, 1.0f) * u;
+  if (gs.fn == JLLM_GATE_GELU_TANH) {
+    const float inner = 0.7978845608028654f * (z + 0.044715f * z * z * z);
+    if (FAST) return z * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-2.8853900817779268f * inner)) * u;  // 0.5 (1 + tanh x) = 1 / (1 + exp(-2x))
+    return 0.5f * z * (1.0f + tanhf(inner)) * u;
+  }
+  const float g = fminf(z, gs.limit);
+  const float v = fminf(fmaxf(u, -gs.limit), gs.limit);
+  return sigmoid_times<FAST>(g, JLLM_SWISH_ALPHA) * (v + 1.0f);
 }
 
 // The scale of an RMSNorm from a row's sum of squares: the mean and the sum with eps in fp32, the inverse square root in

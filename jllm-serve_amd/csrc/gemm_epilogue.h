@@ -4,7 +4,7 @@
 // lane l is output column 8 * (e / 4) + (l / 32) * 4 + e % 4 of the 32-column block and output row l % 32 of the
 // 32-row block; a lane owns four consecutive output columns of one row and stores them at once. Epilogues: store
 // (fp32 or bf16), add into the fp32 residual, gated (accumulators [.][0] and [.][1] are gate and up of the same 32
-// outputs: silu(gate) * up). With `split_z` the wave leaves an fp32 partial tile instead (K cut over workgroups;
+// outputs: the gate function of common.h applied to both). With `split_z` the wave leaves an fp32 partial tile instead (K cut over workgroups;
 // a reduction kernel applies bias and epilogue).
 #pragma once
 #include "common.h"
@@ -13,7 +13,7 @@
 template <bool GATED, int FM, int FN, int TBM, int TBN>
 __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[FM][FN], int lane, int wm, int wn, int m0, int n0,
                                               const void* __restrict__ bias, int bias_dtype, void* __restrict__ out,
-                                              int out_dtype, int ldo, int M, int N, int epilogue, float* __restrict__ partial,
+                                              int out_dtype, int ldo, int M, int N, int epilogue, GateSpec gs, float* __restrict__ partial,
                                               int split_z, int n_splits) {
   // epilogue: accumulator element e of lane l is output column 8 * (e / 4) + (l / 32) * 4 + e % 4 of the 32-column
   // block and output row l % 32 of the 32-row block
@@ -71,7 +71,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[FM][FN], int lane,
 #pragma unroll
           for (int c = 0; c < 4; ++c) {
             float x = acc[mi][ni][4 * e4 + c] + bv[ni][e4][c];
-            if (GATED) x = gate_fn<true>(x) * acc[mi][1][4 * e4 + c];
+            if (GATED) x = gated<true>(x, acc[mi][1][4 * e4 + c], gs);
             v[c] = x;
           }
           const size_t o = row + n;
@@ -103,7 +103,7 @@ __device__ __forceinline__ void tile_epilogue(floatx16 (&acc)[FM][FN], int lane,
         for (int c = 0; c < 4; ++c) {
           float x = acc[mi][ni][4 * e4 + c];
           if (bias && n + c < N) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + c) : ldf((const float*)bias, n + c);
-          if (GATED) x = gate_fn<true>(x) * acc[mi][1][4 * e4 + c];
+          if (GATED) x = gated<true>(x, acc[mi][1][4 * e4 + c], gs);
           v[c] = x;
         }
         const size_t o = (size_t)m * ldo + n;

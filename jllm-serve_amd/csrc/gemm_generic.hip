@@ -4,7 +4,7 @@
 // other rows of the batch.
 //
 // Epilogues: 0 store (fp32 or bf16), 1 add into an fp32 matrix (the residual stream), 2 gated:
-// out = silu(A*Wg^T) * (A*Wu^T) with two weight matrices sharing the A tile.
+// out = gate(A*Wg^T, A*Wu^T) (the gate functions of common.h) with two weight matrices sharing the A tile.
 #include "common.h"
 
 #define GBN 64
@@ -33,12 +33,12 @@ __device__ __forceinline__ void load_tile(const T* __restrict__ base, int ld, in
 // bias, gate and store of one output: the same arithmetic in both kernels of this file
 template <bool GATED>
 __device__ __forceinline__ void finish_output(float v, float up, int m, int n, const void* __restrict__ bias, int bias_dtype,
-                                              void* __restrict__ out, int out_dtype, int ldo, int epilogue) {
+                                              void* __restrict__ out, int out_dtype, int ldo, int epilogue, GateSpec gs) {
   if (bias) v += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n) : ldf((const float*)bias, n);
   const size_t o = (size_t)m * ldo + n;
   if (GATED) {
     const float g = v;
-    v = gate_fn<false>(g) * up;
+    v = gated<false>(g, up, gs);
   }
   if (epilogue == 1) {
     ((float*)out)[o] += v;
@@ -56,7 +56,7 @@ template <typename TA, typename TW, bool GATED, int TM>
 __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                            const TW* __restrict__ W2, const void* __restrict__ bias,
                                                            int bias_dtype, void* __restrict__ out, int out_dtype,
-                                                           int ldo, int M, int N, int K, int epilogue) {
+                                                           int ldo, int M, int N, int K, int epilogue, GateSpec gs) {
   constexpr int GBM = 16 * TM;
   __shared__ float As[GBK][GBM + 4];
   __shared__ float Ws[GBK][GBN + 4];
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(256) void gemm_generic_kernel(const TA* __restrict_
     for (int j = 0; j < 4; ++j) {
       const int n = n0 + tx * 4 + j;
       if (n >= N) continue;
-      finish_output<GATED>(acc[i][j], acc2[i][j], m, n, bias, bias_dtype, out, out_dtype, ldo, epilogue);
+      finish_output<GATED>(acc[i][j], acc2[i][j], m, n, bias, bias_dtype, out, out_dtype, ldo, epilogue, gs);
     }
   }
 }
@@ -123,7 +123,7 @@ template <typename TA, typename TW, bool GATED>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A, int lda, const TW* __restrict__ W,
                                                         const TW* __restrict__ W2, const void* __restrict__ bias,
                                                         int bias_dtype, void* __restrict__ out, int out_dtype, int ldo,
-                                                        int M, int N, int K, int epilogue) {
+                                                        int M, int N, int K, int epilogue, GateSpec gs) {
   __shared__ float ws[2][GATED ? 2 : 1][GR_ROWS][GR_WLD];
   __shared__ float as[2][16][GR_ALD];
   const int r = threadIdx.x & (GR_ROWS - 1), q = threadIdx.x / GR_ROWS;  // q = 0 .. 7
@@ -188,37 +188,37 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(const TA* __restrict__ A
   if (n >= N) return;
 #pragma unroll
   for (int i = 0; i < 2; ++i)
-    if (q + 8 * i < M) finish_output<GATED>(acc[i], acc2[i], q + 8 * i, n, bias, bias_dtype, out, out_dtype, ldo, epilogue);
+    if (q + 8 * i < M) finish_output<GATED>(acc[i], acc2[i], q + 8 * i, n, bias, bias_dtype, out, out_dtype, ldo, epilogue, gs);
 }
 
 template <typename TA, typename TW>
 static void launch_rows(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype, void* out,
-                        int out_dtype, int ldo, int M, int N, int K, int epilogue, hipStream_t stream) {
+                        int out_dtype, int ldo, int M, int N, int K, int epilogue, GateSpec gs, hipStream_t stream) {
   dim3 grid((N + GR_ROWS - 1) / GR_ROWS);
   if (W2)
     gemm_rows_kernel<TA, TW, true><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
-                                                             bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                             bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
   else
     gemm_rows_kernel<TA, TW, false><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
-                                                              bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                              bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
 }
 
 #define GEMM_ROWS_MAX 16
 
 extern "C" int jllm_gemm_generic(const void* A, int a_dtype, int lda, const void* W, const void* W2, int w_dtype,
                                  const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M, int N,
-                                 int K, int epilogue, hipStream_t stream) {
+                                 int K, int epilogue, float gate_limit, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0) JLLM_FAIL("gemm: K=%d", K);
   if (lda < K || ldo < N) JLLM_FAIL("gemm: leading dimensions lda=%d K=%d ldo=%d N=%d", lda, K, ldo, N);
-  JLLM_TAKE_GATE("gemm", epilogue);
+  JLLM_TAKE_GATE("gemm", epilogue, gate_limit, gs);
   if (epilogue < 0 || epilogue > 2) JLLM_FAIL("gemm: epilogue %d", epilogue);
   if ((epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm: the gated epilogue needs exactly two weight matrices");
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm: the accumulate epilogue adds into fp32");
   if (M <= GEMM_ROWS_MAX) {
     JLLM_DISPATCH_1(a_dtype, TA, {
       JLLM_DISPATCH_1(w_dtype, TW, {
-        launch_rows<TA, TW>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, stream);
+        launch_rows<TA, TW>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, stream);
       })
     })
     JLLM_CHECK_LAUNCH("gemm_rows");
@@ -231,16 +231,16 @@ extern "C" int jllm_gemm_generic(const void* A, int a_dtype, int lda, const void
     JLLM_DISPATCH_1(w_dtype, TW, {
       if (W2 && tall)
         gemm_generic_kernel<TA, TW, true, 8><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
-                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
       else if (W2)
         gemm_generic_kernel<TA, TW, true, 4><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, bias,
-                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                                        bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
       else if (tall)
         gemm_generic_kernel<TA, TW, false, 8><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
-                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
       else
         gemm_generic_kernel<TA, TW, false, 4><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, bias,
-                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue);
+                                                                         bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs);
     })
   })
   JLLM_CHECK_LAUNCH("gemm_generic");

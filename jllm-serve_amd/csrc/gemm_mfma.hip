@@ -28,7 +28,7 @@ template <bool GATED, int WGM, int WGN, int FM, int FN, bool DEEP>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
-    int epilogue, float* __restrict__ partial) {
+    int epilogue, GateSpec gs, float* __restrict__ partial) {
   static_assert(FN == 2, "a wave's columns are two 32-wide accumulators (gate and up with the gated epilogue)");
   constexpr int NT = WGM * WGN * 64;
   constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
@@ -166,7 +166,7 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
       }
     }
   }
-  tile_epilogue<GATED, FM, FN, TBM, TBN>(acc, lane, wm, wn, m0, n0, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, partial,
+  tile_epilogue<GATED, FM, FN, TBM, TBN>(acc, lane, wm, wn, m0, n0, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, gs, partial,
                                          (int)blockIdx.z, (int)gridDim.z);
 }
 
@@ -232,7 +232,7 @@ int jllm_splitk_reduce(const float* partial, int splits, const void* bias, int b
 
 template <int WGM, int WGN, int FM, int FN, bool DEEP>
 static int launch_tiled(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
-                        void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int splits,
+                        void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, GateSpec gs, int splits,
                         float* partial, hipStream_t stream) {
   constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
   const int cols = W2 ? TBN / 2 : TBN;
@@ -248,10 +248,10 @@ static int launch_tiled(const void* A, int lda, const void* W, const void* W2, c
   }
   if (W2)
     gemm_mfma_kernel<true, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
   else
     gemm_mfma_kernel<false, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
   return 0;
 }
 
@@ -259,11 +259,11 @@ static int launch_tiled(const void* A, int lda, const void* W, const void* W2, c
 // returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
 extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                    int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
-                                   int splits, float* partial, hipStream_t stream) {
+                                   float gate_limit, int splits, float* partial, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % TBK) || (lda & 7)) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
-  JLLM_TAKE_GATE("gemm_mfma", epilogue);
+  JLLM_TAKE_GATE("gemm_mfma", epilogue, gate_limit, gs);
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_mfma: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_mfma: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_mfma: ldo %d < N %d", ldo, N);
@@ -274,7 +274,7 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   const long big_tiles = (long)((N + (W2 ? 127 : 255)) / (W2 ? 128 : 256)) * ((M + 255) / 256);
   int rc;
   if (splits == 1 && (big_tiles >= 512 || (big_tiles >= 192 && big_tiles <= 256)))
-    rc = launch_tiled<2, 4, 4, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, 1, partial, stream);
+    rc = launch_tiled<2, 4, 4, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, 1, partial, stream);
   else {
     // The small tile with two K steps requested ahead where every workgroup has a compute unit to itself: then a step
     // takes 0.85 us instead of 1.1 (gate/up at 128 rows of the 8B shape, 192 workgroups: 68 -> 54 us; down, 256: 38 ->
@@ -283,9 +283,9 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
     const long groups = (long)((N + (W2 ? 63 : 127)) / (W2 ? 64 : 128)) * ((M + 127) / 128) * splits;
     const int cus = jllm_compute_units();
     if (cus > 0 && groups <= cus)
-      rc = launch_tiled<2, 2, 2, 2, true>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+      rc = launch_tiled<2, 2, 2, 2, true>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, splits, partial, stream);
     else
-      rc = launch_tiled<2, 2, 2, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+      rc = launch_tiled<2, 2, 2, 2, false>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, splits, partial, stream);
   }
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_mfma");

@@ -42,7 +42,7 @@ template <bool GATED, int FM, int NS>
 __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
-    int epilogue, float* __restrict__ partial) {
+    int epilogue, GateSpec gs, float* __restrict__ partial) {
   constexpr int WGM = 2, WGN = 4, FN = 2;
   constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
   constexpr int STAGE = (TBM + TBN) * PP_ROW_BYTES;
@@ -209,13 +209,13 @@ __global__ __launch_bounds__(PP_WAVES * 64) void gemm_pingpong_kernel(
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
   }
-  tile_epilogue<GATED, FM, FN, TBM, TBN>(acc, lane, wm, wn, m0, n0, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, partial,
+  tile_epilogue<GATED, FM, FN, TBM, TBN>(acc, lane, wm, wn, m0, n0, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, gs, partial,
                                          (int)blockIdx.z, (int)gridDim.z);
 }
 
 template <int FM, int NS>
 static int launch_pingpong(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
-                           void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int splits,
+                           void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, GateSpec gs, int splits,
                            float* partial, hipStream_t stream) {
   constexpr int TBM = 2 * FM * 32, TBN = 256;
   const int cols = W2 ? TBN / 2 : TBN;
@@ -231,10 +231,10 @@ static int launch_pingpong(const void* A, int lda, const void* W, const void* W2
   }
   if (W2)
     gemm_pingpong_kernel<true, FM, NS><<<grid, PP_WAVES * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
   else
     gemm_pingpong_kernel<false, FM, NS><<<grid, PP_WAVES * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
   return 0;
 }
 
@@ -243,11 +243,11 @@ static int launch_pingpong(const void* A, int lda, const void* W, const void* W2
 // in ascending order of the split by the other tiled kernel's reduction. Returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors.
 extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                        int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                       int epilogue, int tile_rows, int splits, float* partial, hipStream_t stream) {
+                                       int epilogue, float gate_limit, int tile_rows, int splits, float* partial, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (K <= 0 || (K % PP_BK) || (lda & 7)) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
-  JLLM_TAKE_GATE("gemm_pingpong", epilogue);
+  JLLM_TAKE_GATE("gemm_pingpong", epilogue, gate_limit, gs);
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_pingpong: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_pingpong: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_pingpong: ldo %d < N %d", ldo, N);
@@ -258,7 +258,7 @@ extern "C" int jllm_gemm_pingpong_bf16(const void* A, int lda, const void* W, co
   if (splits > 65535 || (K / PP_BK) / splits < 4) return 1;
   int rc;
   if (tile_rows == 256)
-    rc = launch_pingpong<4, 4>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, splits, partial, stream);
+    rc = launch_pingpong<4, 4>(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, splits, partial, stream);
   else
     JLLM_FAIL("gemm_pingpong: tile of %d rows (256 is built)", tile_rows);
   if (rc != 0) return rc;

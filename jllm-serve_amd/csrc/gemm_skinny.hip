@@ -30,6 +30,7 @@ struct SkinnyNorm {
   const float* norm_partial;  // normed: [M][norm_parts] sums of squares of the input rows
   int norm_parts;
   float norm_eps;
+  GateSpec gate;              // the gate function of the gated epilogue
 };
 
 // sum over the 16 lanes of a row of lanes (the 16 columns of a tile), left in all of them
@@ -323,7 +324,7 @@ __global__ __launch_bounds__(SK_WAVES * 64) void gemm_skinny_kernel(
     for (int i = 0; i < 4; ++i) {
       const int m = mt * 16 + g * 4 + i;
       float v = acc[mt][i] * rscale[mt][i] + b;
-      if (GATED) v = gate_fn<false>(v) * (acc2[mt][i] * rscale[mt][i]);
+      if (GATED) v = gated<false>(v, acc2[mt][i] * rscale[mt][i], nm.gate);
       const float now = prev[mt][i] + v;
       if (nm.emit_rows) {  // every lane of the row takes part in the sum, rows beyond M with zeros
         const float sq = row16_sum(m < M ? now * now : 0.f) + (TWO ? sq2[i] : 0.f);
@@ -370,12 +371,14 @@ static void launch_skinny_mt(int mt, dim3 grid, hipStream_t stream, const void* 
 }
 
 static int skinny_checked(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
-                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, const SkinnyNorm& nm,
-                          int rows2, hipStream_t stream) {
+                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, float gate_limit,
+                          const SkinnyNorm& nm_in, int rows2, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
-  JLLM_TAKE_GATE("gemm_skinny", epilogue);
+  JLLM_TAKE_GATE("gemm_skinny", epilogue, gate_limit, gs);
+  SkinnyNorm nm = nm_in;
+  nm.gate = gs;
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_skinny: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_skinny: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_skinny: ldo %d < N %d", ldo, N);
@@ -421,17 +424,17 @@ static int skinny_checked(const void* A, int lda, const void* W, const void* W2,
 // kernel), -1 on errors
 extern "C" int jllm_gemm_skinny_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                      int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                     int epilogue, int rows2, hipStream_t stream) {
-  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, SkinnyNorm{}, rows2, stream);
+                                     int epilogue, float gate_limit, int rows2, hipStream_t stream) {
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gate_limit, SkinnyNorm{}, rows2, stream);
 }
 
 // The same with an RMSNorm on either side (see the head of this file). emit_rows [M, N] bf16, emit_gain [N] and
 // emit_partial [M][N / 16] fp32 go with the accumulate epilogue; norm_partial [M][norm_parts] with any.
 extern "C" int jllm_gemm_skinny_norm_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                           int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                          int epilogue, int rows2, void* emit_rows, const void* emit_gain,
+                                          int epilogue, float gate_limit, int rows2, void* emit_rows, const void* emit_gain,
                                           int emit_gain_dtype, float* emit_partial, const float* norm_partial,
                                           int norm_parts, float norm_eps, hipStream_t stream) {
-  SkinnyNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps};
-  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, nm, rows2, stream);
+  SkinnyNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps, GateSpec{0, 0.f}};
+  return skinny_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gate_limit, nm, rows2, stream);
 }

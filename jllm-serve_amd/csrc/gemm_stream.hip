@@ -25,7 +25,7 @@ template <int MT, bool GATED>
 __global__ __launch_bounds__(GS_WAVES * 64) void gemm_stream_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
-    int epilogue, float* __restrict__ partial, int blocks_per_part) {
+    int epilogue, GateSpec gs, float* __restrict__ partial, int blocks_per_part) {
   constexpr int UB = GATED ? 1 : 2;            // 128-wide K blocks per step
   constexpr int LD = UB * 128 + 8;             // LDS row stride in elements
   constexpr int PIECES = MT * 16 * UB * 16;    // 16-byte pieces of an activation chunk
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(GS_WAVES * 64) void gemm_stream_kernel(
       const int m = mt * 16 + g * 4 + i;
       if (m >= M) continue;
       float v = acc[mt][i] + b;
-      if (GATED) v = gate_fn<false>(v) * acc2[mt][i];
+      if (GATED) v = gated<false>(v, acc2[mt][i], gs);
       const size_t o = (size_t)m * ldo + n;
       if (epilogue == 1)
         ((float*)out)[o] += v;
@@ -171,6 +171,7 @@ struct StreamNorm {
   int norm_parts;
   float norm_eps;
   int K;
+  GateSpec gate;  // the gate function of the gated epilogue
 };
 
 // adds the K parts in ascending order and applies bias and epilogue; `mats` = 2: gate and up sums side by side.
@@ -220,7 +221,7 @@ __global__ __launch_bounds__(64) void stream_reduce_kernel(const float* __restri
   for (int e = 0; e < V; ++e) {
     float x = v[e];
     if (bias) x += (bias_dtype == JLLM_BF16) ? ldf((const bf16_t*)bias, n + e) : ldf((const float*)bias, n + e);
-    if (mats == 2) x = gate_fn<false>(x) * (u[e] * scale);
+    if (mats == 2) x = gated<false>(x, u[e] * scale, nm.gate);
     r[e] = x;
   }
   if (nm.emit_rows) {  // epilogue 1; the lanes of 16 consecutive columns add their squares (all lanes take part)
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(64) void stream_reduce_kernel(const float* __restri
 template <int MT>
 static void launch_stream(dim3 grid, hipStream_t stream, const void* A, int lda, const void* W, const void* W2,
                           const void* bias, int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                          int epilogue, float* partial, int bpp) {
+                          int epilogue, GateSpec gs, float* partial, int bpp) {
   const size_t smem_g = (size_t)2 * MT * 16 * (128 + 8) * sizeof(bf16_t), smem_p = (size_t)2 * MT * 16 * (256 + 8) * sizeof(bf16_t);
   static bool configured = false;
   if (!configured) {  // above 64 KB the size has to be allowed first
@@ -272,20 +273,22 @@ static void launch_stream(dim3 grid, hipStream_t stream, const void* A, int lda,
   if (W2)
     gemm_stream_kernel<MT, true><<<grid, GS_WAVES * 64, smem_g, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                           (const bf16_t*)W2, bias, bias_dtype, out,
-                                                                          out_dtype, ldo, M, N, K, epilogue, partial, bpp);
+                                                                          out_dtype, ldo, M, N, K, epilogue, gs, partial, bpp);
   else
     gemm_stream_kernel<MT, false><<<grid, GS_WAVES * 64, smem_p, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W,
                                                                            nullptr, bias, bias_dtype, out, out_dtype, ldo,
-                                                                           M, N, K, epilogue, partial, bpp);
+                                                                           M, N, K, epilogue, gs, partial, bpp);
 }
 
 static int stream_checked(const void* A, int lda, const void* W, const void* W2, const void* bias, int bias_dtype,
-                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, int parts, float* partial,
-                          const StreamNorm& nm, hipStream_t stream) {
+                          void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue, float gate_limit, int parts, float* partial,
+                          const StreamNorm& nm_in, hipStream_t stream) {
   if (M <= 0 || N <= 0) return 0;
   if (M > 64 || (K & 127) || (N & 15) || (lda & 7) || K <= 0) return 1;
   if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
-  JLLM_TAKE_GATE("gemm_stream", epilogue);
+  JLLM_TAKE_GATE("gemm_stream", epilogue, gate_limit, gs);
+  StreamNorm nm = nm_in;
+  nm.gate = gs;
   if (epilogue < 0 || epilogue > 2 || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_stream: epilogue %d", epilogue);
   if (epilogue == 1 && out_dtype != JLLM_F32) JLLM_FAIL("gemm_stream: the accumulate epilogue adds into fp32");
   if (ldo < N) JLLM_FAIL("gemm_stream: ldo %d < N %d", ldo, N);
@@ -306,10 +309,10 @@ static int stream_checked(const void* A, int lda, const void* W, const void* W2,
   dim3 grid((N + GS_COLS - 1) / GS_COLS, used);
   if (grid.y > 65535) return 1;
   switch ((M + 15) / 16) {
-    case 1: launch_stream<1>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial, bpp); break;
-    case 2: launch_stream<2>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial, bpp); break;
-    case 3: launch_stream<3>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial, bpp); break;
-    default: launch_stream<4>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, partial, bpp); break;
+    case 1: launch_stream<1>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, bpp); break;
+    case 2: launch_stream<2>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, bpp); break;
+    case 3: launch_stream<3>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, bpp); break;
+    default: launch_stream<4>(grid, stream, A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, bpp); break;
   }
   JLLM_CHECK_LAUNCH("gemm_stream");
   if (used > 1) {
@@ -330,8 +333,8 @@ static int stream_checked(const void* A, int lda, const void* W, const void* W2,
 // returns 0 when it ran, 1 when the shape is not one it takes (the caller uses another kernel), -1 on errors
 extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                      int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K, int epilogue,
-                                     int parts, float* partial, hipStream_t stream) {
-  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, parts, partial, StreamNorm{},
+                                     float gate_limit, int parts, float* partial, hipStream_t stream) {
+  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gate_limit, parts, partial, StreamNorm{},
                         stream);
 }
 
@@ -339,9 +342,9 @@ extern "C" int jllm_gemm_stream_bf16(const void* A, int lda, const void* W, cons
 // and N % 256 == 0, declines otherwise.
 extern "C" int jllm_gemm_stream_norm_bf16(const void* A, int lda, const void* W, const void* W2, const void* bias,
                                           int bias_dtype, void* out, int out_dtype, int ldo, int M, int N, int K,
-                                          int epilogue, int parts, float* partial, void* emit_rows, const void* emit_gain,
+                                          int epilogue, float gate_limit, int parts, float* partial, void* emit_rows, const void* emit_gain,
                                           int emit_gain_dtype, float* emit_partial, const float* norm_partial,
                                           int norm_parts, float norm_eps, hipStream_t stream) {
-  StreamNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps, K};
-  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, parts, partial, nm, stream);
+  StreamNorm nm{(bf16_t*)emit_rows, emit_gain, emit_gain_dtype, emit_partial, norm_partial, norm_parts, norm_eps, K, GateSpec{0, 0.f}};
+  return stream_checked(A, lda, W, W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gate_limit, parts, partial, nm, stream);
 }

@@ -1,0 +1,201 @@
+// A mixture of experts whose routing is a table: row t's experts are table[token[t]][0 .. top). Everything happens
+// on the device, from the token ids, so a step needs no answer from the GPU before it launches (and can be captured).
+//
+//   moe_route     one workgroup: counts the assignments (row, k) of every expert, lays them out expert by expert in
+//                 `sorted`, and cuts each expert's run into tiles of at most `tile_rows` rows: tiles[i] = (expert,
+//                 first place in `sorted`, rows); the tiles no expert needs have 0 rows
+//   moe_gemm      a grouped product over those tiles: every tile multiplies its rows with its expert's weights
+//                 [N, K]. The first product gathers its input rows by token (assignment / top), applies the gate
+//                 function to the two sums and writes hidden rows in the order of `sorted`; the second reads those
+//                 and writes fp32 rows by assignment, or, with top = 1, adds them straight into the residual rows
+//   moe_combine   residual[t] += weight * sum_k y[t * top + k], k ascending
+//
+// The order of `sorted` within an expert comes from LDS atomics and may differ between runs; no result depends on it
+// (every output is one accumulator over ascending k of its own row and weight row). This file is the fp32 path
+// (plain FMAs) and takes any sizes and fp32 or bf16 operands.
+#include "common.h"
+
+#define MOE_ROUTE_THREADS 1024
+
+__global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table,
+                                                                     int T, int top, int E, int tile_rows, int max_tiles,
+                                                                     int* __restrict__ sorted, int* __restrict__ tiles) {
+  extern __shared__ int sh[];
+  int* count = sh;           // [E]
+  int* start = sh + E;       // [E + 1]
+  int* tile0 = sh + 2 * E + 1;  // [E + 1]
+  int* cursor = sh + 3 * E + 2;  // [E]
+  const int A = T * top;
+  for (int e = threadIdx.x; e < E; e += MOE_ROUTE_THREADS) count[e] = 0, cursor[e] = 0;
+  for (int i = threadIdx.x; i < max_tiles; i += MOE_ROUTE_THREADS) {
+    tiles[3 * i] = 0;
+    tiles[3 * i + 1] = 0;
+    tiles[3 * i + 2] = 0;
+  }
+  __syncthreads();
+  for (int a = threadIdx.x; a < A; a += MOE_ROUTE_THREADS) {
+    const int e = table[(size_t)tokens[a / top] * top + a % top];
+    atomicAdd(&count[e], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int s = 0, t = 0;
+    for (int e = 0; e < E; ++e) {
+      start[e] = s;
+      tile0[e] = t;
+      s += count[e];
+      t += (count[e] + tile_rows - 1) / tile_rows;
+    }
+    start[E] = s;
+    tile0[E] = t;
+  }
+  __syncthreads();
+  for (int a = threadIdx.x; a < A; a += MOE_ROUTE_THREADS) {
+    const int e = table[(size_t)tokens[a / top] * top + a % top];
+    sorted[start[e] + atomicAdd(&cursor[e], 1)] = a;
+  }
+  for (int e = threadIdx.x; e < E; e += MOE_ROUTE_THREADS) {
+    const int c = count[e];
+    for (int k = 0; k * tile_rows < c; ++k) {
+      const int i = tile0[e] + k;
+      if (i >= max_tiles) break;
+      tiles[3 * i] = e;
+      tiles[3 * i + 1] = start[e] + k * tile_rows;
+      tiles[3 * i + 2] = min(tile_rows, c - k * tile_rows);
+    }
+  }
+}
+
+extern "C" int jllm_moe_route(const int* tokens, const int* table, int T, int top, int E, int tile_rows, int max_tiles,
+                              int* sorted, int* tiles, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (top <= 0 || E <= 0 || top > E || tile_rows <= 0) JLLM_FAIL("moe_route: top %d of %d experts, tiles of %d rows", top, E, tile_rows);
+  const long A = (long)T * top;
+  const long need = A / tile_rows + E < A ? A / tile_rows + E : A;
+  if (max_tiles < need) JLLM_FAIL("moe_route: room for %d tiles, %ld may be needed", max_tiles, need);
+  const size_t smem = (size_t)(4 * E + 2) * sizeof(int);
+  if (smem > 64 * 1024) JLLM_FAIL("moe_route: %d experts are more than this kernel's LDS holds", E);
+  moe_route_kernel<<<1, MOE_ROUTE_THREADS, smem, stream>>>(tokens, table, T, top, E, tile_rows, max_tiles, sorted, tiles);
+  JLLM_CHECK_LAUNCH("moe_route");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+#define MG_ROWS 16
+#define MG_COLS 64
+#define MG_K 32
+
+// in_map 0: input row = place in `sorted`; 1: the assignment's token row (sorted[place] / top).
+// out_map 0: output row = place in `sorted`; 1: the assignment (sorted[place]); 2: add weight * v into the fp32 row of
+// the assignment's token (top = 1 only: no two assignments share a row).
+template <typename TA, typename TW, bool GATED>
+__global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
+    const TA* __restrict__ A, int lda, const TW* __restrict__ W, const TW* __restrict__ W2, void* __restrict__ out,
+    int out_dtype, int ldo, int N, int K, const int* __restrict__ sorted, const int* __restrict__ tiles, int top,
+    int in_map, int out_map, float weight, GateSpec gs) {
+  const int tile = blockIdx.y;
+  const int rows = tiles[3 * tile + 2];
+  if (rows == 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  __shared__ float As[MG_K][MG_ROWS + 1];
+  __shared__ float Ws[MG_K][MG_COLS + 4];
+  __shared__ float Us[GATED ? MG_K : 1][MG_COLS + 4];
+  __shared__ int src[MG_ROWS], asg[MG_ROWS];
+  if (threadIdx.x < MG_ROWS) {
+    const int place = first + min((int)threadIdx.x, rows - 1);
+    const int a = sorted[place];
+    asg[threadIdx.x] = a;
+    src[threadIdx.x] = in_map ? a / top : place;
+  }
+  __syncthreads();
+  const int n0 = blockIdx.x * MG_COLS;
+  const TW* w = W + (size_t)e * N * K;
+  const TW* w2 = GATED ? W2 + (size_t)e * N * K : nullptr;
+  const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+  float acc[4] = {}, acc2[4] = {};
+  for (int k0 = 0; k0 < K; k0 += MG_K) {
+    for (int i = threadIdx.x; i < MG_ROWS * MG_K; i += 256) {
+      const int r = i / MG_K, k = i % MG_K;
+      As[k][r] = (r < rows && k0 + k < K) ? ldf(A + (size_t)src[r] * lda, k0 + k) : 0.f;
+    }
+    for (int i = threadIdx.x; i < MG_COLS * MG_K; i += 256) {
+      const int r = i / MG_K, k = i % MG_K;
+      const bool in = n0 + r < N && k0 + k < K;
+      Ws[k][r] = in ? ldf(w + (size_t)(n0 + r) * K, k0 + k) : 0.f;
+      if (GATED) Us[k][r] = in ? ldf(w2 + (size_t)(n0 + r) * K, k0 + k) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < MG_K; ++kk) {
+      const float av = As[kk][ty];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        acc[j] = fmaf(av, Ws[kk][tx * 4 + j], acc[j]);
+        if (GATED) acc2[j] = fmaf(av, Us[kk][tx * 4 + j], acc2[j]);
+      }
+    }
+    __syncthreads();
+  }
+  if (ty >= rows) return;
+  const size_t orow = out_map == 0 ? (size_t)(first + ty) : out_map == 1 ? (size_t)asg[ty] : (size_t)(asg[ty] / top);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + tx * 4 + j;
+    if (n >= N) continue;
+    float v = acc[j];
+    if (GATED) v = gated<false>(v, acc2[j], gs);
+    const size_t o = orow * ldo + n;
+    if (out_map == 2)
+      ((float*)out)[o] += weight * v;
+    else if (out_dtype == JLLM_BF16)
+      stf((bf16_t*)out, o, v);
+    else
+      stf((float*)out, o, v);
+  }
+}
+
+extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const void* W, const void* W2, int w_dtype,
+                                     void* out, int out_dtype, int ldo, int N, int K, const int* sorted, const int* tiles,
+                                     int max_tiles, int tile_rows, int top, int in_map, int out_map, float weight,
+                                     int epilogue, float gate_limit, hipStream_t stream) {
+  if (max_tiles <= 0) return 0;
+  if (N <= 0 || K <= 0 || lda < K || ldo < N) JLLM_FAIL("moe_gemm: N %d K %d lda %d ldo %d", N, K, lda, ldo);
+  if (tile_rows != MG_ROWS) JLLM_FAIL("moe_gemm: this kernel takes tiles of %d rows, the route made %d", MG_ROWS, tile_rows);
+  if (max_tiles > 65535) JLLM_FAIL("moe_gemm: %d tiles are too many for one launch", max_tiles);
+  JLLM_TAKE_GATE("moe_gemm", epilogue, gate_limit, gs);
+  if ((epilogue != 0 && epilogue != 2) || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("moe_gemm: epilogue %d", epilogue);
+  if (in_map < 0 || in_map > 1 || out_map < 0 || out_map > 2) JLLM_FAIL("moe_gemm: maps %d / %d", in_map, out_map);
+  if (out_map == 2 && (top != 1 || out_dtype != JLLM_F32)) JLLM_FAIL("moe_gemm: adding into the token's row needs top = 1 and fp32 rows");
+  dim3 grid((N + MG_COLS - 1) / MG_COLS, max_tiles);
+  JLLM_DISPATCH_1(a_dtype, TA, {
+    JLLM_DISPATCH_1(w_dtype, TW, {
+      if (W2)
+        moe_gemm_generic_kernel<TA, TW, true><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, (const TW*)W2, out, out_dtype,
+                                                                        ldo, N, K, sorted, tiles, top, in_map, out_map, weight, gs);
+      else
+        moe_gemm_generic_kernel<TA, TW, false><<<grid, 256, 0, stream>>>((const TA*)A, lda, (const TW*)W, nullptr, out, out_dtype, ldo,
+                                                                         N, K, sorted, tiles, top, in_map, out_map, weight, gs);
+    })
+  })
+  JLLM_CHECK_LAUNCH("moe_gemm_generic");
+  return 0;
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
+                                                         int top, float weight) {
+  const int t = blockIdx.x;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) s += y[((size_t)t * top + k) * width + i];
+    residual[(size_t)t * width + i] += weight * s;
+  }
+}
+
+extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, hipStream_t stream) {
+  if (T <= 0) return 0;
+  if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight);
+  JLLM_CHECK_LAUNCH("moe_combine");
+  return 0;
+}

@@ -20,7 +20,7 @@ F32, BF16 = 0, 1
 EPI_STORE, EPI_ADD, EPI_GATED = 0, 1, 2
 # gate functions of the gated epilogue by name; the code rides in bits 8 and up of the kernels' epilogue argument
 # (csrc/common.h), and a kernel refuses a code it was not built with
-GATE_FUNCTIONS = {"silu": 0}
+GATE_FUNCTIONS = {"silu": 0, "gelu_tanh": 1, "swish_clamped": 2}  # "swish_clamped" takes a limit (``gate_limit``)
 
 
 class KernelError(RuntimeError):
@@ -60,7 +60,7 @@ def _declare(lib) -> None:
     sig = {
         "jllm_embed": [_P, _I, _P, _P, _I, _I, _F, _P],
         "jllm_rmsnorm": [_P, _P, _I, _I, _P, _I, _F, _P, _I, _I, _P],
-        "jllm_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _P],
         "jllm_qk_norm_rope_store": [_P, _I, _I, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P],
         "jllm_paged_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
         "jllm_argmax": [_P, _I, _I, _I, _P, _P, _P],
@@ -68,6 +68,12 @@ def _declare(lib) -> None:
         "jllm_adjust_logits": [_P, _I, _P, _P, _I, _F, _F, _F, _P, _P, _I, _P],
         "jllm_token_logprobs": [_P, _I, _I, _I, _P, _I, _P, _P, _P, _P],
         "jllm_copy_words": [_P, _P, _L, _P],
+        "jllm_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P],
+        "jllm_latent_heads_generic": [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
+        "jllm_latent_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
+        "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P],
+        "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
+        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
     }
     for name, args in sig.items():
@@ -88,16 +94,17 @@ def _declare(lib) -> None:
 
 
 _OPTIONAL_SIGS = {
-    "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P],
-    "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _F, _P],
-    "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
-    "jllm_gemm_pingpong_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P],
-    "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P],
-    "jllm_gemm_stream_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _F, _P],
+    "jllm_gemm_skinny_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "jllm_gemm_skinny_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _P, _P, _I, _F, _P],
+    "jllm_gemm_mfma_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+    "jllm_gemm_pingpong_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _I, _P, _P],
+    "jllm_gemm_stream_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P],
+    "jllm_gemm_stream_norm_bf16": [_P, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _P, _I, _P, _P, _I, _F, _P],
     "jllm_decode_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
 
@@ -255,7 +262,8 @@ class NormedRows:
         return self._rows
 
 
-def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[NormedRows] = None) -> bool:
+def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[NormedRows] = None,
+                 gate_limit: float = 0.0) -> bool:
     """The weight-streaming products (up to 16 rows, up to 64 rows) with a norm on either side; False when the kernel
     does not take the case."""
     M, K = a.shape
@@ -265,7 +273,7 @@ def _skinny_norm(a, w, w2, bias, out, epilogue, emit=None, normed: Optional[Norm
     e_rows, e_gain, e_part = emit if emit is not None else (None, None, None)
     n_part = normed.partials if normed is not None else None
     head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
-            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
+            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue), float(gate_limit))
     tail = (_ptr(e_rows), _ptr(e_gain), _code(e_gain.dtype) if e_gain is not None else F32, _ptr(e_part), _ptr(n_part),
             n_part.shape[1] if n_part is not None else 0, normed.eps if normed is not None else 0.0, _stream())
     few = M <= SKINNY_MAX_ROWS
@@ -304,11 +312,12 @@ def gemm_add_then_norm(a: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gain
 
 def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None, bias: Optional[torch.Tensor] = None,
          out: Optional[torch.Tensor] = None, out_dtype: Optional[torch.dtype] = None, epilogue: int = EPI_STORE,
-         exact: bool = False, gate: int = 0) -> torch.Tensor:
+         exact: bool = False, gate: int = 0, gate_limit: float = 0.0) -> torch.Tensor:
     """out = a @ w.T (+ bias) with ``w`` [N, K] row-major.
 
     EPI_STORE writes ``out_dtype``; EPI_ADD adds into the fp32 ``out`` (the residual stream); EPI_GATED
-    writes gate(a @ w.T) * (a @ w2.T) with the gate function of code ``gate`` (``GATE_FUNCTIONS``; 0 = SiLU).
+    writes gate(a @ w.T, a @ w2.T) with the gate function of code ``gate`` (``GATE_FUNCTIONS``; 0 = SiLU times the
+    second product) and its parameter ``gate_limit`` where it has one.
     ``exact`` forces the plain-FMA fp32-accumulation kernel. ``a`` may be a ``NormedRows``.
     """
     normed = None
@@ -346,16 +355,16 @@ def gemm(a: torch.Tensor, w: torch.Tensor, *, w2: Optional[torch.Tensor] = None,
     if M == 0:
         return out
     if normed is not None:
-        if _skinny_norm(a, w, w2, bias, out, epilogue, normed=normed):
+        if _skinny_norm(a, w, w2, bias, out, epilogue, normed=normed, gate_limit=gate_limit):
             return out
         a = normed.tensor()  # the long way: the norm as a launch of its own
-    if not exact and _fast_gemm is not None and _fast_gemm(a, w, w2, bias, out, epilogue):
+    if not exact and _fast_gemm is not None and _fast_gemm(a, w, w2, bias, out, epilogue, gate_limit):
         return out
     if not exact:
         _count("general", "jllm_gemm_generic")
     _call("jllm_gemm_generic", _ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(bias),
           _code(bias.dtype) if bias is not None else F32, _ptr(out), _code(out.dtype), out.stride(0), M, N, K,
-          int(epilogue), _stream())
+          int(epilogue), float(gate_limit), _stream())
     return out
 
 
@@ -580,7 +589,7 @@ def _few_rows_prefer_stream(N: int, K: int, gated: bool) -> bool:
     return second < 0.95 * first
 
 
-def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
+def _fast_gemm(a, w, w2, bias, out, epilogue, gate_limit: float = 0.0) -> bool:
     """The bf16 matrix-core kernels: a weight-streaming one for up to 16 rows, another for up to 64; for many rows
     the two-group kernel with 256 x 256 tiles where enough of them fill the GPU (`_pingpong_plan`), else the other
     tiled kernel (with K cut over several workgroups when the output has few tiles). Each declines shapes it does
@@ -590,7 +599,7 @@ def _fast_gemm(a, w, w2, bias, out, epilogue) -> bool:
     M, K = a.shape
     N = w.shape[0]
     head = (_ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(bias), _code(bias.dtype) if bias is not None else F32,
-            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue))
+            _ptr(out), _code(out.dtype), out.stride(0), M, N, K, int(epilogue), float(gate_limit))
     if M <= SKINNY_MAX_ROWS and not _few_rows_prefer_stream(N, K, w2 is not None) \
             and _try("jllm_gemm_skinny_bf16", *head, _skinny_second_rows(N, w2 is not None), _stream()):
         return True
@@ -803,6 +812,198 @@ def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
               int(rotary_dim), 1 if write_kv else 0, T, heads, kv_heads, head_dim, k_cache.shape[2], int(window),
               float(scale), max_ctx - 1, _ptr(part_acc), _ptr(part_ml), splits, split, _stream())
     return out if ok else None
+
+
+# ------------------------------------------------------------------------------------------------ latent attention
+
+MAX_LATENT = 512       # the latent a cached row may hold (csrc/latent_generic.hip); the rotated key part comes on top
+
+
+def check_latent_shape(heads: int, kv_rank: int, rot_dim: int, rot_dims: int) -> None:
+    """Raises when no latent-attention kernel takes these sizes; asked when a model is built."""
+    if not 0 < heads <= MAX_HEADS:
+        raise KernelError(f"latent attention: {heads} heads")
+    if not 0 < kv_rank <= MAX_LATENT:
+        raise KernelError(f"latent attention: a latent of {kv_rank} is beyond what the kernels take (1..{MAX_LATENT})")
+    if rot_dim < 0 or rot_dims < 0 or rot_dims > rot_dim or rot_dims % 2:
+        raise KernelError(f"latent attention: {rot_dims} rotated dimensions of a key part of {rot_dim} (even, at most the part)")
+
+
+def _tables(cos, sin, rot_dims):
+    if rot_dims and (cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32
+                     or not cos.is_contiguous() or not sin.is_contiguous() or cos.dim() != 2 or cos.shape != sin.shape
+                     or cos.shape[1] != rot_dims // 2):
+        raise KernelError("rotary tables must be contiguous fp32 [positions, rotary_dim/2]")
+
+
+def latent_prepare(y: torch.Tensor, q_rank: int, gq: torch.Tensor, eps: float, *, kv_off: int = 0, kv_rank: int = 0,
+                   rot_dim: int = 0, rot_dims: int = 0, gkv: Optional[torch.Tensor] = None,
+                   positions: Optional[torch.Tensor] = None, slots: Optional[torch.Tensor] = None,
+                   cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None,
+                   cache: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From the down-projections' output ``y`` [T, ...] (query latent first): the RMS-normed query latent [T, q_rank]
+    (returned), and, with ``cache`` [pages, page_size, kv_rank + rot_dim], the RMS-normed latent y[:, kv_off : kv_off +
+    kv_rank] and the key part behind it, rotated at the rows' positions, stored at the rows' ``slots``."""
+    _dev(y, gq, gkv, positions, slots, cos, sin, cache)
+    _rows2d(y, "latent projections")
+    T = y.shape[0]
+    if gq.numel() != q_rank or not gq.is_contiguous():
+        raise KernelError(f"the query latent's gain has {gq.numel()} entries for {q_rank}")
+    cq = torch.empty((T, q_rank), dtype=y.dtype, device=y.device)
+    if cache is not None:
+        if cache.dtype != y.dtype or not cache.is_contiguous() or cache.dim() != 3 or cache.shape[2] != kv_rank + rot_dim:
+            raise KernelError("the latent cache must be a contiguous [pages, page_size, kv_rank + rot_dim] tensor of the activations' type")
+        if gkv is None or gkv.numel() != kv_rank or not gkv.is_contiguous() or gkv.dtype != gq.dtype:
+            raise KernelError(f"the latent's gain must have {kv_rank} entries of the query gain's type")
+        _i32(positions, T, "positions")
+        _i32(slots, T, "slots")
+        _tables(cos, sin, rot_dims)
+    _call("jllm_latent_prepare", _ptr(y), _code(y.dtype), y.stride(0), T, 0, q_rank, kv_off, kv_rank, rot_dim, rot_dims,
+          _ptr(gq), _ptr(gkv), _code(gq.dtype), float(eps), _ptr(positions), _ptr(slots), _ptr(cos), _ptr(sin), _ptr(cq),
+          cq.stride(0), _ptr(cache), _stream())
+    return cq
+
+
+def latent_heads(x: torch.Tensor, w: torch.Tensor, *, tail: int = 0, rot_dims: int = 0,
+                 positions: Optional[torch.Tensor] = None, cos: Optional[torch.Tensor] = None,
+                 sin: Optional[torch.Tensor] = None, gate: Optional[torch.Tensor] = None, exact: bool = False) -> torch.Tensor:
+    """One product per head in one launch: ``w`` is [H, N, K]; ``x`` [T, H * (K + tail)] holds each head's K inputs
+    followed by ``tail`` more entries. Without ``gate``: out [T, H * (N + tail)], each head's N outputs followed by
+    its tail, the first ``rot_dims`` of it rotated at the rows' positions (the query side of latent attention). With
+    ``gate`` (a [T, H * N] view, ``tail`` 0): out [T, H * N] = product * sigmoid(gate) (the value side)."""
+    _dev(x, w, positions, cos, sin, gate)
+    _rows2d(x, "latent_heads input")
+    if w.dim() != 3 or not w.is_contiguous():
+        raise KernelError("latent_heads weights must be a contiguous [heads, N, K] tensor")
+    H, N, K = w.shape
+    T = x.shape[0]
+    mode = 1 if gate is not None else 0
+    if mode == 1 and tail:
+        raise KernelError("latent_heads: the gated form has no tail")
+    if x.shape[1] != H * (K + tail):
+        raise KernelError(f"latent_heads: rows of {x.shape[1]} for {H} heads of {K} + {tail}")
+    if mode == 0 and tail:
+        _i32(positions, T, "positions")
+        _tables(cos, sin, rot_dims)
+    if gate is not None:
+        _rows2d(gate, "gate rows")
+        if gate.shape != (T, H * N) or gate.dtype != x.dtype:
+            raise KernelError(f"latent_heads: gate rows are {tuple(gate.shape)}, expected {(T, H * N)} of the input's type")
+    out = torch.empty((T, H * (N + tail)), dtype=x.dtype, device=x.device)
+    if T == 0:
+        return out
+    if not exact and _fast_latent_heads(x, w, out, H, N, K, mode, tail, rot_dims, positions, cos, sin, gate):
+        return out
+    if not exact:
+        _count("general", "jllm_latent_heads_generic")
+    _call("jllm_latent_heads_generic", _ptr(x), _code(x.dtype), x.stride(0), K + tail, _ptr(w), _code(w.dtype), _ptr(out),
+          out.stride(0), N + tail, T, H, N, K, mode, tail, rot_dims, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(gate),
+          gate.stride(0) if gate is not None else 0, _stream())
+    return out
+
+
+def _fast_latent_heads(x, w, out, H, N, K, mode, tail, rot_dims, positions, cos, sin, gate) -> bool:
+    return False
+
+
+def latent_attention(qa: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, row_req: torch.Tensor,
+                     positions: torch.Tensor, heads: int, kv_rank: int, window: int, scale: float,
+                     sink: Optional[torch.Tensor], meta=None, exact: bool = False) -> torch.Tensor:
+    """Causal attention of every row of ``qa`` [T, H * Dk] over its request's cached rows [pages, page_size, Dk]: a
+    head's score of a row is its Dk query entries times the row, the values are the rows' first ``kv_rank`` entries;
+    the query at p sees keys p + 1 - window .. p (window 0: all); exp(sink[h]) (fp32, one per head) joins the softmax's
+    denominator. Returns [T, H * kv_rank]."""
+    _dev(qa, cache, block_table, row_req, positions, sink)
+    _rows2d(qa, "latent queries")
+    T = qa.shape[0]
+    if cache.dtype != qa.dtype or not cache.is_contiguous() or cache.dim() != 3:
+        raise KernelError("the latent cache must be a contiguous [pages, page_size, Dk] tensor of the queries' type")
+    Dk = cache.shape[2]
+    if qa.shape[1] != heads * Dk or not 0 < kv_rank <= Dk:
+        raise KernelError(f"latent queries have {qa.shape[1]} entries, expected {heads} x {Dk}")
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block table must be a contiguous int32 [requests, max_blocks] tensor")
+    if sink is not None and (sink.dtype != torch.float32 or sink.numel() != heads or not sink.is_contiguous()):
+        raise KernelError(f"the sinks must be a contiguous fp32 tensor with one entry per head ({heads})")
+    _i32(row_req, T, "row -> request map")
+    _i32(positions, T, "positions")
+    out = torch.empty((T, heads * kv_rank), dtype=qa.dtype, device=qa.device)
+    if T == 0:
+        return out
+    if not exact and _fast_latent_attention(qa, out, cache, block_table, row_req, positions, heads, kv_rank, window, scale, sink, meta):
+        return out
+    if not exact:
+        _count("general", "jllm_latent_attention_generic")
+    _call("jllm_latent_attention_generic", _ptr(qa), qa.stride(0), _ptr(out), out.stride(0), _code(qa.dtype), _ptr(cache),
+          _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads, kv_rank, Dk, cache.shape[1],
+          int(window), float(scale), _ptr(sink), _stream())
+    return out
+
+
+def _fast_latent_attention(qa, out, cache, block_table, row_req, positions, heads, kv_rank, window, scale, sink, meta) -> bool:
+    return False
+
+
+# ------------------------------------------------------------------------------------------------ table-routed experts
+
+MOE_TILE_ROWS = 16     # rows of one expert that a workgroup of the grouped products takes
+
+
+def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
+    """Groups the assignments (row t, k-th expert of its token) by expert, on the device: returns (sorted [T * top]
+    int32: the assignments t * top + k expert by expert; tiles [max_tiles, 3] int32: expert, first place in sorted,
+    rows (0 = unused); max_tiles)."""
+    _dev(token_ids, table)
+    T = token_ids.numel()
+    _i32(token_ids, T, "token ids")
+    if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
+        raise KernelError("the routing table must be a contiguous int32 [vocab, top] tensor")
+    top = table.shape[1]
+    A = T * top
+    max_tiles = max(1, min(A, A // MOE_TILE_ROWS + experts))
+    sorted_ = torch.empty((max(A, 1),), dtype=torch.int32, device=table.device)
+    tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=table.device)
+    _call("jllm_moe_route", _ptr(token_ids), _ptr(table), T, top, experts, MOE_TILE_ROWS, max_tiles, _ptr(sorted_), _ptr(tiles),
+          _stream())
+    return sorted_, tiles, max_tiles
+
+
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optional[torch.Tensor] = None,
+             out: torch.Tensor, in_map: int, out_map: int, weight: float = 1.0, gate: int = 0, gate_limit: float = 0.0,
+             exact: bool = False) -> torch.Tensor:
+    """The grouped product of a routed feed-forward: every tile of ``routing`` multiplies its rows of ``a`` with its
+    expert's weights ``w[e]`` ([experts, N, K]); with ``w2`` the gate function is applied to the two sums. ``in_map``
+    0 / 1: a tile's input rows are its places in the sorted order / its assignments' token rows; ``out_map`` 0 / 1 / 2:
+    output rows by place / by assignment / added, times ``weight``, into the fp32 row of the token (top = 1)."""
+    sorted_, tiles, max_tiles = routing
+    _dev(a, w, w2, out)
+    _rows2d(a, "moe input")
+    _rows2d(out, "moe output")
+    if w.dim() != 3 or not w.is_contiguous() or (w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous())):
+        raise KernelError("moe weights must be contiguous [experts, N, K] tensors of one shape and type")
+    _, N, K = w.shape
+    if a.shape[1] != K or out.shape[1] != N:
+        raise KernelError(f"moe_gemm: rows of {a.shape[1]} -> {out.shape[1]} with weights {tuple(w.shape)}")
+    epilogue = (EPI_GATED | (int(gate) << 8)) if w2 is not None else EPI_STORE
+    head = (_ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(out), _code(out.dtype),
+            out.stride(0), N, K, _ptr(sorted_), _ptr(tiles), max_tiles, MOE_TILE_ROWS, int(top), int(in_map), int(out_map),
+            float(weight), epilogue, float(gate_limit), _stream())
+    if not exact and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _try("jllm_moe_gemm_bf16", *head):
+        return out
+    if not exact:
+        _count("general", "jllm_moe_gemm_generic")
+    _call("jllm_moe_gemm_generic", *head)
+    return out
+
+
+def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float) -> None:
+    """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending)."""
+    _dev(y, residual)
+    T, width = residual.shape
+    if y.dtype != torch.float32 or residual.dtype != torch.float32 or not y.is_contiguous() or not residual.is_contiguous() \
+            or y.shape != (T * top, width):
+        raise KernelError("moe_combine takes contiguous fp32 [T * top, width] rows and the fp32 residual [T, width]")
+    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

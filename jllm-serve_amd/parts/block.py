@@ -17,12 +17,17 @@ from .base import Part, part_factory, register_part
 
 class PreNormBlock(Part):
     def __init__(self, spec, prefix, build, positions):
-        self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}.weight", build)
-        self.norm_post = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_post_name}.weight",
-                                                            build)
+        ending = getattr(spec, "name_ending", ".weight")
+        self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}{ending}", build)
         self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, prefix, build, positions)
-        self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
-        self.parts = (self.norm_in, self.mixer, self.norm_post, self.ffn)
+        if spec.ffn is None:  # a layer of a mixer alone: no second norm, no feed-forward
+            self.norm_post = self.ffn = None
+            self.parts = (self.norm_in, self.mixer)
+        else:
+            self.norm_post = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden,
+                                                                f"{prefix}.{spec.norm_post_name}{ending}", build)
+            self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
+            self.parts = (self.norm_in, self.mixer, self.norm_post, self.ffn)
         self.capturable = all(getattr(p, "capturable", True) for p in self.parts)
 
     def weight_specs(self):
@@ -55,6 +60,11 @@ class PreNormBlock(Part):
         """``normed_in``: norm_in of x, prepared by whoever wrote x last (or None); ``next_norm``: the norm part that
         will read x next. Returns that norm of the new x as a promise when the feed-forward prepared it."""
         xb = self._input(self.norm_in, self.mixer, x, normed_in)
+        if self.ffn is None:
+            if next_norm is not None and getattr(self.mixer, "prepares_next_norm", False) and hasattr(next_norm, "after_add"):
+                return self.mixer.forward(xb, x, step, slot, then_norm=next_norm)
+            self.mixer.forward(xb, x, step, slot)
+            return None
         if getattr(self.mixer, "prepares_next_norm", False) and hasattr(self.norm_post, "after_add"):
             mid = self.mixer.forward(xb, x, step, slot, then_norm=self.norm_post)
         else:

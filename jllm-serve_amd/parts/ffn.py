@@ -1,6 +1,7 @@
-"""Dense gated feed-forward: x += W_down (silu(W_gate xb) * (W_up xb)) (cpu/CpuBackend.java:661-669,
+"""Dense gated feed-forward: x += W_down (act(W_gate xb) * (W_up xb)) (cpu/CpuBackend.java:661-669,
 :1289-1300; tensors model/MlpWeights.java:19-33). The activation and product are the epilogue of the
-gate/up product; the residual add is the epilogue of the down product."""
+gate/up product; the residual add is the epilogue of the down product. The gate function is the spec's
+``activation`` (``ops.GATE_FUNCTIONS``), with the spec's ``limit`` where the function has one."""
 from __future__ import annotations
 
 from ..config.schema import GatedMlpSpec
@@ -17,6 +18,7 @@ class GatedMlp(Part):
             raise ValueError(f"unsupported activation '{spec.activation}': the product kernels have "
                              f"{sorted(ops.GATE_FUNCTIONS)} as gate functions")
         self.gate = ops.GATE_FUNCTIONS[spec.activation]
+        self.limit = float(getattr(spec, "limit", 0.0))
         self.hidden = spec.hidden
         self.names = spec.names
         self.dim = build.hidden
@@ -25,7 +27,7 @@ class GatedMlp(Part):
         self.w_gate = self.w_up = self.w_down = None
 
     def _name(self, which: str) -> str:
-        return f"{self.prefix}.{getattr(self.names, which)}.weight"
+        return f"{self.prefix}.{getattr(self.names, which)}{getattr(self.names, 'ending', '.weight')}"
 
     def weight_specs(self):
         if self.names.gate_up is not None:  # one stacked tensor [gate | up]
@@ -45,7 +47,7 @@ class GatedMlp(Part):
 
     def forward(self, xb, residual, step, then_norm=None):
         h = ops.gemm(xb, self.w_gate, w2=self.w_up, epilogue=ops.EPI_GATED, out_dtype=self.build.dtype,
-                     exact=self.build.exact, gate=self.gate)
+                     exact=self.build.exact, gate=self.gate, gate_limit=self.limit)
         if then_norm is not None:
             return then_norm.after_add(h, self.w_down, residual, exact=self.build.exact)
         ops.gemm(h, self.w_down, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)

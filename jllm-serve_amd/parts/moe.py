@@ -1,0 +1,85 @@
+"""A mixture of experts routed by a table: x += (1 / top) * sum over the token's experts of expert(xb) (+ shared(xb)).
+
+Every token id has ``top`` experts in an integer table [vocab, top]; there is no router. An expert is a gated
+feed-forward with the clamped gate (``ops.GATE_FUNCTIONS["swish_clamped"]``, the spec's ``limit``); a shared expert, when
+the spec has one, is a dense gated feed-forward that runs for every row.
+
+The routing happens on the device from the step's token ids (``ops.moe_route``), the experts' products are grouped
+launches over tiles of rows of one expert (``ops.moe_gemm``): gate/up gathers the rows by token and writes hidden rows
+in expert order; down writes per assignment (summed into the residual by ``ops.moe_combine``) or, with top = 1, adds
+into the residual itself. Nothing waits for the GPU, so a decode step with this feed-forward can be captured.
+"""
+from __future__ import annotations
+
+import torch
+
+from ..config.schema import TableMoeSpec
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import BuildContext, Part, part_factory, register_part
+
+
+class TableMoe(Part):
+    def __init__(self, spec: TableMoeSpec, prefix: str, build: BuildContext):
+        if not 0 < spec.top <= spec.experts:
+            raise ValueError(f"{prefix}: top {spec.top} of {spec.experts} experts")
+        self.spec = spec
+        self.prefix = prefix
+        self.build = build
+        self.gate = ops.GATE_FUNCTIONS["swish_clamped"]
+        self.shared = part_factory("ffn", spec.shared.kind)(spec.shared, prefix, build) if spec.shared is not None else None
+        self.takes_normed_rows = False  # the rows are gathered by the grouped product, not fed to ops.gemm
+        self.w_gate = self.w_up = self.w_down = self.table = None
+
+    def _expert(self, e: int, which: str) -> str:
+        n = self.spec.names
+        return f"{self.prefix}.{n.expert}{e}.{getattr(n, which)}{n.ending}"
+
+    def _table_name(self) -> str:
+        return f"{self.prefix}.{self.spec.names.table}{self.spec.names.ending}"
+
+    def weight_specs(self):
+        s, d = self.spec, self.build.hidden
+        out = []
+        for e in range(s.experts):
+            out += [WeightSpec(self._expert(e, "gate"), (s.hidden, d)), WeightSpec(self._expert(e, "up"), (s.hidden, d)),
+                    WeightSpec(self._expert(e, "down"), (d, s.hidden))]
+        from ..weights.loader import EXPERT_COUNTS
+        EXPERT_COUNTS[self._table_name()] = s.experts  # for the random-weights mode
+        out.append(WeightSpec(self._table_name(), (s.vocab, s.top), init="expert_table"))
+        if self.shared is not None:
+            out += self.shared.weight_specs()
+        return out
+
+    def load(self, get):
+        s = self.spec
+        stack = lambda which: torch.stack([get(self._expert(e, which)) for e in range(s.experts)]).contiguous()
+        self.w_gate, self.w_up, self.w_down = stack("gate"), stack("up"), stack("down")
+        table = get(self._table_name()).to(torch.int32).contiguous()
+        lo, hi = int(table.min()), int(table.max())
+        if lo < 0 or hi >= s.experts:
+            raise ValueError(f"{self._table_name()}: entries {lo}..{hi} for {s.experts} experts")
+        self.table = table
+        if self.shared is not None:
+            self.shared.load(get)
+
+    def forward(self, xb, residual, step, then_norm=None):
+        s, exact = self.spec, self.build.exact
+        T = xb.shape[0]
+        if self.shared is not None:
+            self.shared.forward(xb, residual, step)
+        routing = ops.moe_route(step.token_ids, self.table, s.experts)
+        A = T * s.top
+        hidden = torch.empty((A, s.hidden), dtype=self.build.dtype, device=xb.device)
+        ops.moe_gemm(xb, self.w_gate, routing, s.top, w2=self.w_up, out=hidden, in_map=1, out_map=0, gate=self.gate,
+                     gate_limit=s.limit, exact=exact)
+        if s.top == 1:
+            ops.moe_gemm(hidden, self.w_down, routing, 1, out=residual, in_map=0, out_map=2, weight=1.0, exact=exact)
+        else:
+            y = torch.empty((A, residual.shape[1]), dtype=torch.float32, device=xb.device)
+            ops.moe_gemm(hidden, self.w_down, routing, s.top, out=y, in_map=0, out_map=1, exact=exact)
+            ops.moe_combine(y, residual, s.top, 1.0 / s.top)
+        return None
+
+
+register_part("ffn", "table_moe", TableMoe, replace=True)

@@ -40,7 +40,8 @@ class WeightError(ValueError):
 @dataclass(frozen=True)
 class WeightSpec:
     """One tensor a part needs. ``init`` tells the random-weights mode how to fill it:
-    "matrix" N(0, std), "gain" 1 + N(0, gain_std), "bias" N(0, std), "zeros"."""
+    "matrix" N(0, std), "gain" 1 + N(0, gain_std), "bias" N(0, std), "zeros", "expert_table" (int32 [rows, top]:
+    every row holds ``top`` different expert numbers below the count that the tensor's name is registered with)."""
 
     name: str
     shape: Tuple[int, ...]
@@ -79,6 +80,11 @@ def fetch(source, name: str, run_dtype: torch.dtype, device) -> torch.Tensor:
     if t.dtype != want:
         t = t.to(want)
     return t.contiguous()
+
+
+# how many experts the rows of a routing table may name, by tensor name: a routed feed-forward registers its table here
+# when it declares it, for the random-weights mode
+EXPERT_COUNTS: Dict[str, int] = {}
 
 
 class TensorSource:
@@ -124,7 +130,7 @@ class RandomSource:
         return self.specs[name].shape
 
     def dtype(self, name: str) -> torch.dtype:
-        return self._dtype
+        return torch.int32 if self.specs[name].init == "expert_table" else self._dtype
 
     def get(self, name: str) -> torch.Tensor:
         s = self.specs[name]
@@ -132,6 +138,11 @@ class RandomSource:
         g.manual_seed((self.seed * 1000003 + zlib.crc32(name.encode("utf-8"))) % (2**63 - 1))
         if s.init == "zeros":
             return torch.zeros(s.shape, dtype=self._dtype, device=self.device)
+        if s.init == "expert_table":  # every row: `top` different experts; the count rides in the spec's name table
+            rows, top = s.shape
+            experts = EXPERT_COUNTS.get(name, top)
+            scores = torch.rand((rows, experts), generator=g, dtype=torch.float32, device=self.device)
+            return scores.argsort(dim=1)[:, :top].to(torch.int32).contiguous()
         if s.init == "gain":
             if self.gain_std == 0:
                 return torch.ones(s.shape, dtype=self._dtype, device=self.device)

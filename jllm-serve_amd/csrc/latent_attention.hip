@@ -1,0 +1,199 @@
+// Latent attention on the matrix cores, bf16: portions of prompts and single decoded rows through one kernel.
+//
+// All heads of a row attend over the same cached rows (Dk = R + Dr numbers per position, the first R of which are also
+// the values), so the query vectors of many heads and rows share every key they read. A workgroup of four waves takes
+// 64 query vectors of one run of rows of one request (HB heads x 64 / HB consecutive rows; a wave owns 16 of them),
+// walks the keys its rows can see in blocks of 64 aligned to absolute positions, and stages each block once in LDS as
+// it lies in the cache. Per 16 keys a wave computes
+//   S^T = K . Q^T   (MFMA 16x16x32; K fragments from LDS, Q^T in registers): a lane then holds four keys' scores of
+//                   ONE query vector, so masks (causal and window, per query vector), maximum and sum need only two
+//                   shuffles over the lane groups;
+//   O^T += V^T . P^T (MFMA 16x16x16): those probabilities, packed to bf16, already are the B operand, and V^T is read
+//                   from the staged block with the transposing LDS load.
+// The running maximum moves only when it grows by more than 8 (probabilities stay below e^8, exact in fp32 sums).
+// exp(sink) of the query vector's head joins the denominator at the end. Scores, softmax and sums are fp32.
+//
+// The runs come from the step's plan: (request, first row, rows <= 16, -) per tile; positions are read per row.
+#include <math.h>
+
+#include "common.h"
+#include "mfma.h"
+
+#define LM_WAVES 4
+#define LM_KEYS 64
+#define LM_TILE_ROWS 16
+
+__device__ __forceinline__ float lm_exp_diff(float a, float b) { return a == -INFINITY ? 0.f : __expf(a - b); }
+
+// RT: 16-dim blocks of the latent the accumulators hold at most; DKS: 32-dim steps of a key row at most
+template <int RT, int DKS>
+__global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
+    const bf16_t* __restrict__ qa, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ cache,
+    const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
+    const int* __restrict__ positions, int H, int R, int Dk, int page_size, int window, float scale,
+    const float* __restrict__ sink, int HB, int n_hb, int LD) {
+  extern __shared__ __align__(16) unsigned char lm_smem[];
+  bf16_t* Ks = (bf16_t*)lm_smem;  // [LM_KEYS][LD]
+  const int tile = blockIdx.x;
+  const int req = tiles[4 * tile], row0 = tiles[4 * tile + 1], rows = tiles[4 * tile + 2];
+  const int RW = 64 / HB;
+  const int rg = blockIdx.y / n_hb, hb = blockIdx.y % n_hb;
+  const int r_lo = rg * RW;
+  if (r_lo >= rows) return;
+  const int r_hi = min(rows, r_lo + RW) - 1;
+  const int p_lo = positions[row0 + r_lo];
+  const int p_hi = p_lo + (r_hi - r_lo);
+  const int kb = window > 0 ? max(0, p_lo + 1 - window) : 0;
+  const int ke = p_hi;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int sub = lane & 15, q4 = lane >> 4;
+  const int v = wave * 16 + sub;
+  const int my_r = r_lo + v / HB, my_h = hb * HB + v % HB;
+  const bool live = my_r <= r_hi && my_h < H;
+  const int my_pos = p_lo + v / HB;
+  const int my_first = window > 0 ? max(0, my_pos + 1 - window) : 0;
+  // the keys this wave's rows can see (a wave without a live query vector only helps to load)
+  const int wr_lo = r_lo + (wave * 16) / HB, wr_hi = min(r_hi, r_lo + (wave * 16 + 15) / HB);
+  const bool wave_live = wr_lo <= r_hi;
+  const int w_lo = window > 0 ? max(0, p_lo + (wr_lo - r_lo) + 1 - window) : 0;
+  const int w_hi = p_lo + (wr_hi - r_lo);
+  const int dks = (Dk + 31) >> 5, r16 = R >> 4;
+  const int psh = __builtin_ctz(page_size);
+  const int* tbl = block_table + (size_t)req * max_blocks;
+
+  u32x4 qf[DKS];
+  {
+    const bf16_t* qrow = qa + (size_t)(row0 + min(my_r, r_hi)) * ldq + (size_t)min(my_h, H - 1) * Dk;
+#pragma unroll
+    for (int j = 0; j < DKS; ++j) {
+      const int d = 32 * j + 8 * q4;
+      qf[j] = (live && j < dks && d < Dk) ? *(const u32x4*)(qrow + d) : u32x4{0u, 0u, 0u, 0u};
+    }
+  }
+  floatx4 acc[RT];
+#pragma unroll
+  for (int j = 0; j < RT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  float m1 = -INFINITY, l1 = 0.f;
+  const int chunks = dks * 4;  // 16-byte pieces of a staged row (zero beyond Dk)
+
+  for (int blk = kb >> 6; blk <= (ke >> 6); ++blk) {
+    const int c0 = blk * LM_KEYS;
+    __syncthreads();  // everyone is done with the block before
+    for (int idx = threadIdx.x; idx < LM_KEYS * chunks; idx += LM_WAVES * 64) {
+      const int r = idx / chunks, c = idx - r * chunks;
+      const int key = min(max(c0 + r, kb), ke);  // a key outside the range is masked below and reads one inside it
+      const int page = tbl[key >> psh];
+      uint4 val = uint4{0u, 0u, 0u, 0u};
+      if (8 * c < Dk) val = *(const uint4*)(cache + ((((size_t)page) << psh) + (key & (page_size - 1))) * Dk + 8 * c);
+      *(uint4*)(Ks + r * LD + 8 * c) = val;
+    }
+    __syncthreads();
+    if (!wave_live) continue;
+#pragma unroll 1
+    for (int st = 0; st < LM_KEYS / 16; ++st) {
+      const int k0 = c0 + st * 16;
+      if (k0 + 15 < w_lo || k0 > w_hi) continue;  // none of these keys is seen by a row of this wave
+      floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
+      const bf16_t* krow = Ks + (st * 16 + sub) * LD + 8 * q4;
+#pragma unroll
+      for (int j = 0; j < DKS; ++j)
+        if (j < dks) sc = mfma16(*(const u32x4*)(krow + 32 * j), qf[j], sc);
+      float z[4];
+      float mx = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int key = k0 + 4 * q4 + i;
+        z[i] = (live && key >= my_first && key <= my_pos) ? sc[i] * scale : -INFINITY;
+        mx = fmaxf(mx, z[i]);
+      }
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      if (mx > m1 + 8.0f) {  // also the first visible key (m1 = -inf)
+        const float alpha = lm_exp_diff(m1, mx);
+        l1 *= alpha;
+#pragma unroll
+        for (int j = 0; j < RT; ++j) acc[j] *= alpha;
+        m1 = mx;
+      }
+      float p[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[i] = lm_exp_diff(z[i], m1);
+        l1 += p[i];
+      }
+      const u32x2 pb = u32x2{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3])};
+      const bf16_t* v_tr = Ks + (st * 16 + 4 * q4 + (sub >> 2)) * LD + 4 * (sub & 3);
+#pragma unroll
+      for (int j = 0; j < RT; ++j)
+        if (j < r16) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * j), pb, acc[j]);
+    }
+  }
+  if (!live) return;
+  l1 += __shfl_xor(l1, 16, 64);
+  l1 += __shfl_xor(l1, 32, 64);
+  float ca = 1.0f;
+  if (sink) {
+    const float sk = sink[my_h];
+    const float mn = fmaxf(m1, sk);
+    ca = lm_exp_diff(m1, mn);
+    l1 = l1 * ca + __expf(sk - mn);
+  }
+  const float inv = ca / l1;
+  bf16_t* o = out + (size_t)(row0 + my_r) * ldo + (size_t)my_h * R + 4 * q4;
+#pragma unroll
+  for (int j = 0; j < RT; ++j)
+    if (j < r16)
+      *(u32x2*)(o + 16 * j) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
+}
+
+template <int RT, int DKS>
+static int lm_launch(dim3 grid, size_t smem, hipStream_t stream, const void* qa, int ldq, void* out, int ldo, const void* cache,
+                     const int* block_table, int max_blocks, const int* tiles, const int* positions, int H, int R, int Dk,
+                     int page_size, int window, float scale, const float* sink, int HB, int n_hb, int LD) {
+  static size_t reserved = 0;
+  if (smem > 48 * 1024 && smem > reserved) {
+    if (hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RT, DKS>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)smem) != hipSuccess)
+      JLLM_FAIL("latent_attention: cannot reserve %zu bytes of LDS", smem);
+    reserved = smem;
+  }
+  latent_attention_mfma_kernel<RT, DKS><<<grid, LM_WAVES * 64, smem, stream>>>(
+      (const bf16_t*)qa, ldq, (bf16_t*)out, ldo, (const bf16_t*)cache, block_table, max_blocks, tiles, positions, H, R, Dk,
+      page_size, window, scale, sink, HB, n_hb, LD);
+  return 0;
+}
+
+// returns 0 when it ran, 1 when the shape is not one it takes (the caller uses the general kernel), -1 on errors
+extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, int ldo, const void* cache,
+                                          const int* block_table, int max_blocks, const int* tiles, const int* positions,
+                                          int n_tiles, int tile_rows, int H, int R, int Dk, int page_size, int window,
+                                          float scale, const float* sink, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (tile_rows != LM_TILE_ROWS) JLLM_FAIL("latent_attention: runs of %d rows, this kernel takes %d", tile_rows, LM_TILE_ROWS);
+  if (H <= 0 || R <= 0 || Dk < R || window < 0 || page_size <= 0 || max_blocks <= 0) JLLM_FAIL("latent_attention: H %d R %d Dk %d window %d", H, R, Dk, window);
+  if ((R & 15) || (Dk & 7) || R > 512 || Dk > 640 || (page_size & (page_size - 1))) return 1;
+  if (((uintptr_t)qa & 15) || ((uintptr_t)cache & 15) || ((uintptr_t)out & 7) || (ldq & 7) || (ldo & 3)) return 1;
+  if (ldq < H * Dk || ldo < H * R) JLLM_FAIL("latent_attention: row strides %d/%d", ldq, ldo);
+  int HB = 1;
+  while (HB < H && HB < 64) HB <<= 1;
+  const int RW = 64 / HB;
+  const int n_hb = (H + HB - 1) / HB, n_rg = (LM_TILE_ROWS + RW - 1) / RW;
+  if ((long)n_hb * n_rg > 65535) return 1;
+  // staged rows lie (Dk rounded up to 32) + pad elements apart, with the stride = 16 mod 64 elements (8 mod 32 words):
+  // four consecutive rows of a transposing load then cover all banks
+  const int dkp = (Dk + 31) & ~31;
+  int LD = dkp + 16;
+  while ((LD & 63) != 16) LD += 8;
+  const size_t smem = (size_t)LM_KEYS * LD * sizeof(bf16_t);
+  dim3 grid(n_tiles, n_hb * n_rg);
+  int rc;
+  if (R <= 64 && dkp <= 128)
+    rc = lm_launch<4, 4>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+  else if (R <= 128 && dkp <= 256)
+    rc = lm_launch<8, 8>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+  else
+    rc = lm_launch<32, 20>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+  if (rc != 0) return rc;
+  JLLM_CHECK_LAUNCH("latent_attention");
+  return 0;
+}

@@ -104,6 +104,8 @@ _OPTIONAL_SIGS = {
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P],
+    "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -903,7 +905,12 @@ def latent_heads(x: torch.Tensor, w: torch.Tensor, *, tail: int = 0, rot_dims: i
 
 
 def _fast_latent_heads(x, w, out, H, N, K, mode, tail, rot_dims, positions, cos, sin, gate) -> bool:
-    return False
+    """The bf16 matrix-core kernel; it declines shapes whose rows do not start on 16-byte boundaries."""
+    if x.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+        return False
+    return _try("jllm_latent_heads_bf16", _ptr(x), x.stride(0), K + tail, _ptr(w), _ptr(out), out.stride(0), N + tail,
+                x.shape[0], H, N, K, mode, tail, rot_dims, _ptr(positions), _ptr(cos), _ptr(sin), _ptr(gate),
+                gate.stride(0) if gate is not None else 0, _stream())
 
 
 def latent_attention(qa: torch.Tensor, cache: torch.Tensor, block_table: torch.Tensor, row_req: torch.Tensor,
@@ -940,8 +947,18 @@ def latent_attention(qa: torch.Tensor, cache: torch.Tensor, block_table: torch.T
     return out
 
 
+LATENT_TILE_ROWS = 16  # rows of one request per run of the step's plan (parts/latent_attention.py)
+
+
 def _fast_latent_attention(qa, out, cache, block_table, row_req, positions, heads, kv_rank, window, scale, sink, meta) -> bool:
-    return False
+    """The bf16 matrix-core kernel, for portions and single rows alike; it needs the step's runs of rows (``meta``:
+    ``tiles_dev``, ``n_tiles``) and declines sizes it does not take."""
+    if qa.dtype != torch.bfloat16 or meta is None or meta.get("tiles_dev") is None:
+        return False
+    return _try("jllm_latent_attention_bf16", _ptr(qa), qa.stride(0), _ptr(out), out.stride(0), _ptr(cache),
+                _ptr(block_table), block_table.shape[1], _ptr(meta["tiles_dev"]), _ptr(positions), int(meta["n_tiles"]),
+                LATENT_TILE_ROWS, heads, kv_rank, cache.shape[2], cache.shape[1], int(window), float(scale), _ptr(sink),
+                _stream())
 
 
 # ------------------------------------------------------------------------------------------------ table-routed experts

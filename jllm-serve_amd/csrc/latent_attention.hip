@@ -14,6 +14,10 @@
 // exp(sink) of the query vector's head joins the denominator at the end. Scores, softmax and sums are fp32.
 //
 // The runs come from the step's plan: (request, first row, rows <= 16, -) per tile; positions are read per row.
+//
+// Steps of single rows (decoding) with few workgroups cut every row's keys into absolute ranges of `split` keys over
+// gridDim.z: a workgroup then leaves maximum, sum and unnormalised sums per query vector, and a second kernel merges
+// the ranges in ascending order, adds the sink and normalises.
 #include <math.h>
 
 #include "common.h"
@@ -31,7 +35,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
     const bf16_t* __restrict__ qa, int ldq, bf16_t* __restrict__ out, int ldo, const bf16_t* __restrict__ cache,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ positions, int H, int R, int Dk, int page_size, int window, float scale,
-    const float* __restrict__ sink, int HB, int n_hb, int LD) {
+    const float* __restrict__ sink, int HB, int n_hb, int LD, int split, float* __restrict__ part) {
   extern __shared__ __align__(16) unsigned char lm_smem[];
   bf16_t* Ks = (bf16_t*)lm_smem;  // [LM_KEYS][LD]
   const int tile = blockIdx.x;
@@ -43,8 +47,14 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   const int r_hi = min(rows, r_lo + RW) - 1;
   const int p_lo = positions[row0 + r_lo];
   const int p_hi = p_lo + (r_hi - r_lo);
-  const int kb = window > 0 ? max(0, p_lo + 1 - window) : 0;
-  const int ke = p_hi;
+  int kb = window > 0 ? max(0, p_lo + 1 - window) : 0;
+  int ke = p_hi;
+  if (split > 0) {  // single rows: this workgroup's range of the row's keys
+    const int s0 = kb / split + (int)blockIdx.z;
+    kb = max(kb, s0 * split);
+    ke = min(ke, s0 * split + split - 1);
+    if (kb > ke) return;
+  }
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int sub = lane & 15, q4 = lane >> 4;
   const int v = wave * 16 + sub;
@@ -56,7 +66,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   const int wr_lo = r_lo + (wave * 16) / HB, wr_hi = min(r_hi, r_lo + (wave * 16 + 15) / HB);
   const bool wave_live = wr_lo <= r_hi;
   const int w_lo = window > 0 ? max(0, p_lo + (wr_lo - r_lo) + 1 - window) : 0;
-  const int w_hi = p_lo + (wr_hi - r_lo);
+  const int w_hi = p_lo + (wr_hi - r_lo);  // (with a split the loop's own bounds narrow these further)
   const int dks = (Dk + 31) >> 5, r16 = R >> 4;
   const int psh = __builtin_ctz(page_size);
   const int* tbl = block_table + (size_t)req * max_blocks;
@@ -131,6 +141,14 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   if (!live) return;
   l1 += __shfl_xor(l1, 16, 64);
   l1 += __shfl_xor(l1, 32, 64);
+  if (split > 0) {
+    float* dst = part + (((size_t)(row0 + my_r) * H + my_h) * gridDim.z + blockIdx.z) * (R + 4);  // R sums, maximum, sum
+    if (q4 == 0) dst[R] = m1, dst[R + 1] = l1;
+#pragma unroll
+    for (int j = 0; j < RT; ++j)
+      if (j < r16) *(floatx4*)(dst + 16 * j + 4 * q4) = acc[j];
+    return;
+  }
   float ca = 1.0f;
   if (sink) {
     const float sk = sink[my_h];
@@ -146,10 +164,52 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       *(u32x2*)(o + 16 * j) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
 }
 
+// merges the key ranges of one (row, head) in ascending order; one wave per (row, head)
+__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part, const int* __restrict__ positions,
+                                                                   int H, int R, int window, int split, int n_z,
+                                                                   const float* __restrict__ sink, bf16_t* __restrict__ out,
+                                                                   int ldo) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int pos = positions[t];
+  const int first = window > 0 ? max(0, pos + 1 - window) : 0;
+  const int s0 = first / split;
+  float m = -INFINITY, l = 0.f;
+  float acc[8];  // R <= 512
+#pragma unroll
+  for (int a = 0; a < 8; ++a) acc[a] = 0.f;
+  for (int z = 0; z < n_z; ++z) {
+    if ((s0 + z) * split > pos) break;
+    const float* src = part + (((size_t)t * H + h) * n_z + z) * (R + 4);
+    const float pm = src[R], pl = src[R + 1];
+    const float mn = fmaxf(m, pm);
+    const float ca = lm_exp_diff(m, mn), cb = lm_exp_diff(pm, mn);
+    l = l * ca + pl * cb;
+#pragma unroll
+    for (int a = 0; a < 8; ++a) {
+      const int d = lane + 64 * a;
+      if (d < R) acc[a] = acc[a] * ca + src[d] * cb;
+    }
+    m = mn;
+  }
+  float ca = 1.0f;
+  if (sink) {
+    const float sk = sink[h];
+    const float mn = fmaxf(m, sk);
+    ca = lm_exp_diff(m, mn);
+    l = l * ca + __expf(sk - mn);
+  }
+  const float inv = ca / l;
+#pragma unroll
+  for (int a = 0; a < 8; ++a) {
+    const int d = lane + 64 * a;
+    if (d < R) stf(out + (size_t)t * ldo + (size_t)h * R, d, acc[a] * inv);
+  }
+}
+
 template <int RT, int DKS>
 static int lm_launch(dim3 grid, size_t smem, hipStream_t stream, const void* qa, int ldq, void* out, int ldo, const void* cache,
                      const int* block_table, int max_blocks, const int* tiles, const int* positions, int H, int R, int Dk,
-                     int page_size, int window, float scale, const float* sink, int HB, int n_hb, int LD) {
+                     int page_size, int window, float scale, const float* sink, int HB, int n_hb, int LD, int split, float* part) {
   static size_t reserved = 0;
   if (smem > 48 * 1024 && smem > reserved) {
     if (hipFuncSetAttribute((const void*)latent_attention_mfma_kernel<RT, DKS>, hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -159,7 +219,7 @@ static int lm_launch(dim3 grid, size_t smem, hipStream_t stream, const void* qa,
   }
   latent_attention_mfma_kernel<RT, DKS><<<grid, LM_WAVES * 64, smem, stream>>>(
       (const bf16_t*)qa, ldq, (bf16_t*)out, ldo, (const bf16_t*)cache, block_table, max_blocks, tiles, positions, H, R, Dk,
-      page_size, window, scale, sink, HB, n_hb, LD);
+      page_size, window, scale, sink, HB, n_hb, LD, split, part);
   return 0;
 }
 
@@ -167,7 +227,8 @@ static int lm_launch(dim3 grid, size_t smem, hipStream_t stream, const void* qa,
 extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, int ldo, const void* cache,
                                           const int* block_table, int max_blocks, const int* tiles, const int* positions,
                                           int n_tiles, int tile_rows, int H, int R, int Dk, int page_size, int window,
-                                          float scale, const float* sink, hipStream_t stream) {
+                                          float scale, const float* sink, int split, int n_z, float* part,
+                                          hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (tile_rows != LM_TILE_ROWS) JLLM_FAIL("latent_attention: runs of %d rows, this kernel takes %d", tile_rows, LM_TILE_ROWS);
   if (H <= 0 || R <= 0 || Dk < R || window < 0 || page_size <= 0 || max_blocks <= 0) JLLM_FAIL("latent_attention: H %d R %d Dk %d window %d", H, R, Dk, window);
@@ -185,15 +246,22 @@ extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, in
   int LD = dkp + 16;
   while ((LD & 63) != 16) LD += 8;
   const size_t smem = (size_t)LM_KEYS * LD * sizeof(bf16_t);
-  dim3 grid(n_tiles, n_hb * n_rg);
+  // `split` > 0: every tile is a single row (the caller's promise), whose keys are cut into absolute ranges of `split`
+  // keys over n_z workgroups; `part` holds rows x H x n_z x (R + 4) floats
+  if (split > 0 && ((split & 63) || n_z < 1 || n_z > 65535 || !part)) JLLM_FAIL("latent_attention: ranges of %d keys over %d workgroups", split, n_z);
+  dim3 grid(n_tiles, n_hb * (split > 0 ? 1 : n_rg), split > 0 ? n_z : 1);
   int rc;
   if (R <= 64 && dkp <= 128)
-    rc = lm_launch<4, 4>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+    rc = lm_launch<4, 4>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD, split, part);
   else if (R <= 128 && dkp <= 256)
-    rc = lm_launch<8, 8>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+    rc = lm_launch<8, 8>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD, split, part);
   else
-    rc = lm_launch<32, 20>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD);
+    rc = lm_launch<32, 20>(grid, smem, stream, qa, ldq, out, ldo, cache, block_table, max_blocks, tiles, positions, H, R, Dk, page_size, window, scale, sink, HB, n_hb, LD, split, part);
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("latent_attention");
+  if (split > 0) {
+    latent_attention_merge_kernel<<<dim3(n_tiles, H), 64, 0, stream>>>(part, positions, H, R, window, split, n_z, sink, (bf16_t*)out, ldo);
+    JLLM_CHECK_LAUNCH("latent_attention_merge");
+  }
   return 0;
 }

@@ -104,7 +104,7 @@ _OPTIONAL_SIGS = {
     "jllm_decode_attention_fused_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _P, _P, _P, _P, _P, _I, _F, _I, _I, _I, _I, _I,
                                          _I, _I, _I, _F, _I, _P, _P, _I, _I, _P],
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
-    "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _P],
+    "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
@@ -955,10 +955,33 @@ def _fast_latent_attention(qa, out, cache, block_table, row_req, positions, head
     ``tiles_dev``, ``n_tiles``) and declines sizes it does not take."""
     if qa.dtype != torch.bfloat16 or meta is None or meta.get("tiles_dev") is None:
         return False
+    n_tiles = int(meta["n_tiles"])
+    split, n_z, part = 0, 1, None
+    if meta.get("single_rows") and n_tiles == qa.shape[0]:
+        split, n_z = _latent_split(n_tiles, heads, int(window), int(meta.get("max_context", 0)))
+        if split:
+            part = torch.empty((n_tiles * heads * n_z * (kv_rank + 4),), dtype=torch.float32, device=qa.device)
     return _try("jllm_latent_attention_bf16", _ptr(qa), qa.stride(0), _ptr(out), out.stride(0), _ptr(cache),
-                _ptr(block_table), block_table.shape[1], _ptr(meta["tiles_dev"]), _ptr(positions), int(meta["n_tiles"]),
+                _ptr(block_table), block_table.shape[1], _ptr(meta["tiles_dev"]), _ptr(positions), n_tiles,
                 LATENT_TILE_ROWS, heads, kv_rank, cache.shape[2], cache.shape[1], int(window), float(scale), _ptr(sink),
-                _stream())
+                split, n_z, _ptr(part), _stream())
+
+
+LATENT_SPLIT_MIN = 128  # keys a workgroup takes at least when a row's keys are cut over several
+
+
+def _latent_split(rows: int, heads: int, window: int, max_ctx: int):
+    """(keys per range, ranges per row) for a step of single rows, or (0, 1): a row's keys are cut over several
+    workgroups where the step would otherwise leave most compute units idle (few rows, long spans). From the number of
+    rows, the heads, the window and the longest context only (what a captured step's bucket fixes)."""
+    span = min(window, max_ctx) if window > 0 else max_ctx
+    groups = rows * -(-heads // 64)
+    want = -(-2 * compute_units() // max(groups, 1))
+    if span < 2 * LATENT_SPLIT_MIN or want < 2:
+        return 0, 1
+    split = max(LATENT_SPLIT_MIN, -(-(-(-span // want)) // 64) * 64)
+    n_z = -(-span // split) + 1  # a span of that many keys touches at most this many absolute ranges
+    return (split, n_z) if n_z > 2 else (0, 1)
 
 
 # ------------------------------------------------------------------------------------------------ table-routed experts

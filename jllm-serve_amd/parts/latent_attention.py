@@ -46,7 +46,8 @@ class LatentStepPlanner:
             runs = [(s.index, s.row0 + r, min(TILE_ROWS, s.n - r), s.pos0 + r) for s in batch.segments
                     for r in range(0, s.n, TILE_ROWS)]
             runs.sort(key=lambda t: -(t[3] + t[2]))
-        return StepPlan({"tiles": [v for t in runs for v in t]}, {"n_tiles": len(runs)})
+        single = batch.padded or all(s.n == 1 for s in batch.segments)
+        return StepPlan({"tiles": [v for t in runs for v in t]}, {"n_tiles": len(runs), "single_rows": single})
 
 
 class LatentAttention(Part):

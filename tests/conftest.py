@@ -38,3 +38,13 @@ def plain_logits(model_folders):
             cache[key] = tiny.plain_forward(model_folders[name], tokens)
         return cache[key]
     return get
+
+
+@pytest.fixture(scope="session")
+def miforax_folders(tmp_path_factory):
+    """Model folders of the tiny Miforax configurations, made once."""
+    import miforax_tiny
+    out = {}
+    for name, (cfg, seed, page) in miforax_tiny.CONFIGS.items():
+        out[name] = miforax_tiny.write_model(str(tmp_path_factory.mktemp("miforax_" + name)), cfg, seed)
+    return out

@@ -17,6 +17,11 @@ request sets served to the end, with the time the roofline allows for their pass
 `--no-serve`, `--no-fp32`, `--no-long` and `--no-shapes` leave groups out; `--temperature/--top-k/--top-p` make the
 main decode run a sampled one.
 
+`--workload compare [--size 2k|4k]` is another run altogether: a Miforax model (latent attention with a window, dense
+and table-routed expert layers in turn) beside the closest model the engine had before, a Qwen3 dense model with the
+same width, layers, heads, window and feed-forward width, both with random weights: prefill of 2,048 tokens and
+decoding at batch 8 and 64 with full windows, each with the fraction of the published peaks behind it.
+
 A decode step must read every weight once and the keys and values of the live requests: bytes = weights + KV bytes
 per token x tokens held (mean over the timed steps). A prefill must do 2 flops per weight and row, plus 4 x heads x
 head size per (row, key) pair and layer, plus the head for the rows whose logits are wanted.
@@ -65,9 +70,17 @@ class Work:
         self.layer_params = (self.H * self.hd + 2 * self.Hkv * self.hd) * self.d + self.d * self.H * self.hd + 3 * self.d * self.F
         self.weight_bytes = (self.L * self.layer_params + self.V * self.d) * self.esize
         self.kv_bytes_per_token = 2 * self.L * self.Hkv * self.hd * self.esize
+        self.window = shape.get("sliding_window", 0) if shape.get("use_sliding_window") else 0
 
-    def decode_bytes(self, tokens_held: float) -> float:
+    def decode_bytes(self, tokens_held: float, batch: int = 0) -> float:
+        if self.window and batch:  # a request reads no more keys than its window holds
+            tokens_held = min(tokens_held, float(self.window) * batch)
         return self.weight_bytes + self.kv_bytes_per_token * tokens_held
+
+    def pairs(self, T: int) -> float:
+        """(row, key) pairs of one prompt of T tokens from position 0."""
+        w = self.window or T
+        return sum(min(i + 1, w) for i in range(T))
 
     def flops(self, rows: float, pairs: float, selected: float) -> float:
         """``rows`` through every layer, ``pairs`` of (row, key) in the attention of every layer, ``selected`` rows
@@ -81,6 +94,101 @@ class Work:
         by = self.weight_bytes + self.kv_bytes_per_token * one_keys
         fl = self.flops(ones + rows, one_keys + pairs, ones + (1 if rows else 0))
         return max(by / HBM_PEAK, fl / FLOP_PEAK[self.dtype])
+
+
+COMPARE_SIZES = {  # layer sizes that resemble released models with latent attention and routed experts
+    "2k": dict(width=2048, layers=4, heads=16, dim=128, rot=64, vdim=128, q_rank=768, kv_rank=512, window=1024, ff=8192,
+               experts=32, top=4, expert_ff=1024, shared_ff=4096, kv_heads=8, vocab=32768),
+    "4k": dict(width=4096, layers=4, heads=32, dim=128, rot=64, vdim=128, q_rank=1536, kv_rank=512, window=4096, ff=12288,
+               experts=64, top=6, expert_ff=1536, shared_ff=3072, kv_heads=8, vocab=32768),
+}
+
+
+def miforax_config(z: dict) -> dict:
+    """Layers of latent attention with a window; dense and expert feed-forwards in turn, the experts sized so that a
+    token passes through as many feed-forward weights as in a dense layer (top x expert_ff + shared_ff = ff)."""
+    mixer = {"heads": z["heads"], "dim": z["dim"], "rot_dim": z["rot"], "vdim": z["vdim"], "q_rank": z["q_rank"],
+             "kv_rank": z["kv_rank"], "scale": (z["dim"] + z["rot"]) ** -0.5, "mask": {"size": z["window"]},
+             "rot": {"base": 1e6, "dims": z["rot"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
+    dense = {"kind": "dense", "ff": z["ff"]}
+    moe = {"kind": "moe", "router": {"experts": z["experts"], "top": z["top"]}, "expert": {"ff": z["expert_ff"], "limit": 7.0},
+           "shared": {"ff": z["shared_ff"], "limit": 7.0}}
+    return {"architecture": "Miforax", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+            "max_positions": 8192,
+            "layers": [{"type": "latent_attention", "mixer": mixer, "mlp": moe if i % 2 else dense} for i in range(z["layers"])]}
+
+
+def qwen_like_config(z: dict) -> dict:
+    return dict(model_type="qwen3", architectures=["Qwen3ForCausalLM"], num_hidden_layers=z["layers"], hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"], intermediate_size=z["ff"],
+                vocab_size=z["vocab"], rope_theta=1e6, rms_norm_eps=1e-6, tie_word_embeddings=False, max_position_embeddings=8192,
+                use_sliding_window=True, sliding_window=z["window"], max_window_layers=0)
+
+
+class LatentWork:
+    """Bytes and flops of passes over a Miforax model of the sizes ``z`` (the interface of ``Work``). A decode step
+    reads every weight outside the experts, of the experts at most batch x top per layer, and per request the cached
+    rows its window holds; a row costs 2 flops per weight it passes through (of the experts: top), and per (row, key)
+    pair and head 2 x (kv_rank + rot) for the score and 2 x kv_rank for the weighted sum."""
+
+    def __init__(self, z: dict, dtype: str):
+        self.z = z
+        self.L, self.d, self.H, self.Hkv, self.F, self.V = z["layers"], z["width"], z["heads"], 1, z["ff"], z["vocab"]
+        self.hd = z["kv_rank"] + z["rot"]
+        self.window = z["window"]
+        self.esize = 2 if dtype == "bf16" else 4
+        self.dtype = dtype
+        d, H, r = self.d, self.H, z["kv_rank"]
+        self.mixer = (z["q_rank"] + r + z["rot"] + H * z["vdim"]) * d + H * (z["dim"] + z["rot"]) * z["q_rank"] \
+            + H * z["dim"] * r + H * z["vdim"] * r + d * H * z["vdim"]
+        self.dense_ff = 3 * d * z["ff"]
+        self.shared_ff = 3 * d * z["shared_ff"]
+        self.expert = 3 * d * z["expert_ff"]
+        self.n_moe = self.L // 2
+        self.n_dense = self.L - self.n_moe
+        self.kv_bytes_per_token = self.L * self.hd * self.esize
+        self.weight_bytes = (self.L * self.mixer + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + z["experts"] * self.expert)
+                             + self.V * d) * self.esize
+
+    def decode_bytes(self, tokens_held: float, batch: int = 0) -> float:
+        z = self.z
+        touched = min(z["experts"], max(batch, 1) * z["top"])
+        w = (self.L * self.mixer + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + touched * self.expert) + self.V * self.d)
+        if batch:
+            tokens_held = min(tokens_held, float(self.window) * batch)
+        return w * self.esize + self.kv_bytes_per_token * tokens_held
+
+    def pairs(self, T: int) -> float:
+        return sum(min(i + 1, self.window) for i in range(T))
+
+    def flops(self, rows: float, pairs: float, selected: float) -> float:
+        per_row = self.L * self.mixer + self.n_dense * self.dense_ff + self.n_moe * (self.shared_ff + self.z["top"] * self.expert)
+        return 2.0 * rows * per_row + 2.0 * self.H * (self.hd + self.z["kv_rank"]) * self.L * pairs + 2.0 * self.V * self.d * selected
+
+
+def compare_workload(args) -> dict:
+    """``--workload compare``: the Miforax model of ``--size`` and the Qwen3 dense model of the same sizes, one after
+    the other: prefill of 2,048 tokens in one portion, decoding at batch 8 and 64 with every window full."""
+    z = COMPARE_SIZES[args.size]
+    ctx = z["window"] + 1024
+    decodes = [dict(key=f"b{B}", batch=B, prompt_len=z["window"] + 128, steps=args.point_steps, warmup=4) for B in (8, 64)]
+    prefills = [dict(key="main", tokens=2048, portion=2048)]
+    out = {"metric": f"Miforax beside Qwen3 dense at equal sizes ({args.size})", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "higher_is_better": True,
+           "config": {"size": args.size, **z, "context": ctx, "page_size": PAGE}, "models": {}}
+    for name, shape, work in (("miforax", miforax_config(z), LatentWork(z, "bf16")),
+                              ("qwen3_dense", qwen_like_config(z), None)):
+        r = steady(args, name, "bf16", 0, ctx, decodes, prefills, shape=shape, work=work)
+        m = {"prefill_2048_tok_s": r["prefill"]["main"]["value"], "prefill_2048_ms": r["prefill"]["main"]["ms"],
+             "prefill_flop_frac": r["prefill"]["main"]["frac"]}
+        for B in (8, 64):
+            s_, held, by = r["decode"][f"b{B}"]
+            m[f"decode_b{B}_tok_s"] = round(B / s_, 1)
+            m[f"decode_b{B}_ms"] = round(s_ * 1e3, 3)
+            m[f"decode_b{B}_hbm_frac"] = round(by / s_ / HBM_PEAK, 4)
+        out["models"][name] = m
+    out["value"] = out["models"]["miforax"]["decode_b8_tok_s"]
+    return out
 
 
 def sampling_of(args, max_tokens: int):
@@ -201,8 +309,10 @@ def main() -> int:
     ap.add_argument("--no-long", action="store_true", help="steady: leave out the long-context and sampled points")
     ap.add_argument("--no-shapes", action="store_true", help="steady: leave out steady decoding at the 14B and 32B shapes")
     ap.add_argument("--fp32-layers", type=int, default=4, help="layers of the float32 run (named in config)")
-    ap.add_argument("--workload", default="steady", choices=["steady", "serve"],
-                    help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end")
+    ap.add_argument("--workload", default="steady", choices=["steady", "serve", "compare"],
+                    help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end; "
+                         "compare: a Miforax model beside the Qwen3 dense model of the same sizes")
+    ap.add_argument("--size", default="2k", choices=sorted(COMPARE_SIZES), help="compare: which sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -210,6 +320,9 @@ def main() -> int:
 
     if args.workload == "serve":
         print(json.dumps(serve_workload(args)))
+        return 0
+    if args.workload == "compare":
+        print(json.dumps(compare_workload(args)))
         return 0
 
     import torch
@@ -323,11 +436,12 @@ def main() -> int:
     return 0
 
 
-def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes, prefills) -> dict:
+def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes, prefills, shape=None, work=None) -> dict:
     """Builds the shape with random weights in ``dtype`` ("bf16" or "fp32") and measures prefills (``tokens`` of one
     prompt in portions of ``portion``, through the step function) and steady decoding (``batch`` requests with prompts
     of ``prompt_len``, through the engine's loop): {"prefill": {key: {...}}, "decode": {key: (s per step, tokens held
-    on average, bytes a step must read)}, "config": {...}}."""
+    on average, bytes a step must read)}, "config": {...}}. ``shape`` / ``work``: a config.json dict of any registered
+    architecture and the object that prices its passes, in place of the named Qwen3 shape's."""
     import torch
     from jllm_serve_amd.config import parse_config
     from jllm_serve_amd.engine import Engine, SchedulerConfig, build_model, build_runner
@@ -336,9 +450,11 @@ def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes
     from jllm_serve_amd.weights.random_init import random_source
 
     dev = torch.device("cuda:0")
-    shape = shape_config(shape_name)
-    full_layers = shape["num_hidden_layers"]
-    if layers:
+    given = shape is not None
+    if not given:
+        shape = shape_config(shape_name)
+    full_layers = shape["num_hidden_layers"] if "num_hidden_layers" in shape else len(shape["layers"])
+    if layers and not given:
         shape["num_hidden_layers"] = layers
     cfg = parse_config(shape)
     run_dtype = "bfloat16" if dtype == "bf16" else "float32"
@@ -347,7 +463,7 @@ def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes
     model = build_model(cfg, source, run_dtype, dev, context)
     torch.cuda.synchronize()
     print(f"[bench] {dtype} model built in {time.time() - t0:.0f} s: {cfg.description}", file=sys.stderr, flush=True)
-    work = Work(shape, dtype)
+    work = work or Work(shape, dtype)
     chunk = 2048
 
     def held(p):  # positions a request of this point holds at most, in whole pages of 64
@@ -391,7 +507,7 @@ def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes
             once()
         sync()
         s_ = (time.perf_counter() - t) / reps
-        flops = work.flops(T, T * (T + 1) / 2, 1)
+        flops = work.flops(T, work.pairs(T), 1)
         prefill[p["key"]] = {"value": round(T / s_, 1), "tokens": T, "ms": round(s_ * 1e3, 3),
                              "frac": round(flops / s_ / FLOP_PEAK[dtype], 4), "flops": flops}
         print(f"[bench] {shape_name} {dtype} prefill {T} tokens in portions of {portion}: {s_ * 1e3:.1f} ms "
@@ -427,12 +543,12 @@ def steady(args, shape_name: str, dtype: str, layers: int, context: int, decodes
     results = {}
     for p in decodes:
         step_s, held_mean = decode(p)
-        by = work.decode_bytes(held_mean)
+        by = work.decode_bytes(held_mean, p["batch"])
         results[p["key"]] = (step_s, held_mean, by)
         print(f"[bench] {shape_name} {dtype} decode {p['key']}: batch {p['batch']}, {held_mean / p['batch']:.0f} keys each: "
               f"{step_s * 1e3:.2f} ms/step = {p['batch'] / step_s:.1f} tok/s, {by / step_s / 1e12:.2f} TB/s",
               file=sys.stderr, flush=True)
-    config = {"model": f"Qwen3-{shape_name.upper()} shape", "layers": work.L, "layers_in_shape": full_layers, "hidden": work.d,
+    config = {"model": f"Qwen3-{shape_name.upper()} shape" if not given else cfg.description, "layers": work.L, "layers_in_shape": full_layers, "hidden": work.d,
               "heads": work.H, "kv_heads": work.Hkv, "head_dim": work.hd, "intermediate": work.F, "vocab": V,
               "batch": args.batch, "prompt_len": args.prompt_len, "context": context, "page_size": PAGE,
               "global_batch": args.batch, "seq_len": args.prompt_len, "parallelism": "single GPU"}

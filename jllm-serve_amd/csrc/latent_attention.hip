@@ -4,7 +4,7 @@
 // the values), so the query vectors of many heads and rows share every key they read. A workgroup of four waves takes
 // 64 query vectors of one run of rows of one request (HB heads x 64 / HB consecutive rows; a wave owns 16 of them),
 // walks the keys its rows can see in blocks of 64 aligned to absolute positions, and stages each block once in LDS as
-// it lies in the cache. Per 16 keys a wave computes
+// it lies in the cache (two buffers take turns: the next block travels while this one is multiplied). Per 16 keys a wave computes
 //   S^T = K . Q^T   (MFMA 16x16x32; K fragments from LDS, Q^T in registers): a lane then holds four keys' scores of
 //                   ONE query vector, so masks (causal and window, per query vector), maximum and sum need only two
 //                   shuffles over the lane groups;
@@ -37,7 +37,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
     const int* __restrict__ positions, int H, int R, int Dk, int page_size, int window, float scale,
     const float* __restrict__ sink, int HB, int n_hb, int LD, int split, float* __restrict__ part) {
   extern __shared__ __align__(16) unsigned char lm_smem[];
-  bf16_t* Ks = (bf16_t*)lm_smem;  // [LM_KEYS][LD]
+  bf16_t* Ks = (bf16_t*)lm_smem;  // [2][LM_KEYS][LD]
   const int tile = blockIdx.x;
   const int req = tiles[4 * tile], row0 = tiles[4 * tile + 1], rows = tiles[4 * tile + 2];
   const int RW = 64 / HB;
@@ -85,58 +85,93 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   for (int j = 0; j < RT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m1 = -INFINITY, l1 = 0.f;
   const int chunks = dks * 4;  // 16-byte pieces of a staged row (zero beyond Dk)
-
-  for (int blk = kb >> 6; blk <= (ke >> 6); ++blk) {
+  // A block of 64 keys goes global -> registers -> LDS. All of a thread's pieces are requested together (first their
+  // table entries, then the rows: two latencies a block, not two per piece), and the next block's are requested before
+  // this block is multiplied, into the other of two LDS buffers: one barrier per block.
+  constexpr int CPT = (LM_KEYS * DKS * 4 + LM_WAVES * 64 - 1) / (LM_WAVES * 64);
+  uint4 staged[CPT];
+  auto fetch = [&](int blk) {
     const int c0 = blk * LM_KEYS;
-    __syncthreads();  // everyone is done with the block before
-    for (int idx = threadIdx.x; idx < LM_KEYS * chunks; idx += LM_WAVES * 64) {
+    int page[CPT];
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int idx = threadIdx.x + LM_WAVES * 64 * i;
+      const int key = min(max(c0 + idx / chunks, kb), ke);  // a key outside the range is masked below and reads one inside it
+      page[i] = tbl[key >> psh];
+    }
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int idx = threadIdx.x + LM_WAVES * 64 * i;
       const int r = idx / chunks, c = idx - r * chunks;
-      const int key = min(max(c0 + r, kb), ke);  // a key outside the range is masked below and reads one inside it
-      const int page = tbl[key >> psh];
-      uint4 val = uint4{0u, 0u, 0u, 0u};
-      if (8 * c < Dk) val = *(const uint4*)(cache + ((((size_t)page) << psh) + (key & (page_size - 1))) * Dk + 8 * c);
-      *(uint4*)(Ks + r * LD + 8 * c) = val;
+      const int key = min(max(c0 + r, kb), ke);
+      staged[i] = uint4{0u, 0u, 0u, 0u};
+      if (idx < LM_KEYS * chunks && 8 * c < Dk)
+        staged[i] = *(const uint4*)(cache + ((((size_t)page[i]) << psh) + (key & (page_size - 1))) * Dk + 8 * c);
     }
-    __syncthreads();
-    if (!wave_live) continue;
+  };
+  auto put = [&](bf16_t* buf) {
+#pragma unroll
+    for (int i = 0; i < CPT; ++i) {
+      const int idx = threadIdx.x + LM_WAVES * 64 * i;
+      const int r = idx / chunks, c = idx - r * chunks;
+      if (idx < LM_KEYS * chunks) *(uint4*)(buf + r * LD + 8 * c) = staged[i];
+    }
+  };
+  const int blk_last = ke >> 6;
+  int cur = 0;
+  fetch(kb >> 6);
+  put(Ks);
+  __syncthreads();
+  for (int blk = kb >> 6; blk <= blk_last; ++blk) {
+    const int c0 = blk * LM_KEYS;
+    const bf16_t* Kb = Ks + (size_t)cur * LM_KEYS * LD;
+    if (blk < blk_last) fetch(blk + 1);
+    if (wave_live) {
 #pragma unroll 1
-    for (int st = 0; st < LM_KEYS / 16; ++st) {
-      const int k0 = c0 + st * 16;
-      if (k0 + 15 < w_lo || k0 > w_hi) continue;  // none of these keys is seen by a row of this wave
-      floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f};
-      const bf16_t* krow = Ks + (st * 16 + sub) * LD + 8 * q4;
+      for (int st = 0; st < LM_KEYS / 16; ++st) {
+        const int k0 = c0 + st * 16;
+        if (k0 + 15 < w_lo || k0 > w_hi) continue;  // none of these keys is seen by a row of this wave
+        floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f}, sc2 = floatx4{0.f, 0.f, 0.f, 0.f};  // two chains of dependent MFMAs
+        const bf16_t* krow = Kb + (st * 16 + sub) * LD + 8 * q4;
 #pragma unroll
-      for (int j = 0; j < DKS; ++j)
-        if (j < dks) sc = mfma16(*(const u32x4*)(krow + 32 * j), qf[j], sc);
-      float z[4];
-      float mx = -INFINITY;
+        for (int j = 0; j < DKS; j += 2) {
+          if (j < dks) sc = mfma16(*(const u32x4*)(krow + 32 * j), qf[j], sc);
+          if (j + 1 < DKS && j + 1 < dks) sc2 = mfma16(*(const u32x4*)(krow + 32 * (j + 1)), qf[j + 1 < DKS ? j + 1 : j], sc2);
+        }
+        sc += sc2;
+        float z[4];
+        float mx = -INFINITY;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = k0 + 4 * q4 + i;
-        z[i] = (live && key >= my_first && key <= my_pos) ? sc[i] * scale : -INFINITY;
-        mx = fmaxf(mx, z[i]);
+        for (int i = 0; i < 4; ++i) {
+          const int key = k0 + 4 * q4 + i;
+          z[i] = (live && key >= my_first && key <= my_pos && key >= kb && key <= ke) ? sc[i] * scale : -INFINITY;
+          mx = fmaxf(mx, z[i]);
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        if (mx > m1 + 8.0f) {  // also the first visible key (m1 = -inf)
+          const float alpha = lm_exp_diff(m1, mx);
+          l1 *= alpha;
+#pragma unroll
+          for (int j = 0; j < RT; ++j) acc[j] *= alpha;
+          m1 = mx;
+        }
+        float p[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          p[i] = lm_exp_diff(z[i], m1);
+          l1 += p[i];
+        }
+        const u32x2 pb = u32x2{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3])};
+        const bf16_t* v_tr = Kb + (st * 16 + 4 * q4 + (sub >> 2)) * LD + 4 * (sub & 3);
+#pragma unroll
+        for (int j = 0; j < RT; ++j)
+          if (j < r16) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * j), pb, acc[j]);
       }
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      if (mx > m1 + 8.0f) {  // also the first visible key (m1 = -inf)
-        const float alpha = lm_exp_diff(m1, mx);
-        l1 *= alpha;
-#pragma unroll
-        for (int j = 0; j < RT; ++j) acc[j] *= alpha;
-        m1 = mx;
-      }
-      float p[4];
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[i] = lm_exp_diff(z[i], m1);
-        l1 += p[i];
-      }
-      const u32x2 pb = u32x2{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3])};
-      const bf16_t* v_tr = Ks + (st * 16 + 4 * q4 + (sub >> 2)) * LD + 4 * (sub & 3);
-#pragma unroll
-      for (int j = 0; j < RT; ++j)
-        if (j < r16) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * j), pb, acc[j]);
     }
+    if (blk < blk_last) put(Ks + (size_t)(cur ^ 1) * LM_KEYS * LD);
+    __syncthreads();  // the other buffer is whole, and everyone is done with this one
+    cur ^= 1;
   }
   if (!live) return;
   l1 += __shfl_xor(l1, 16, 64);
@@ -245,7 +280,7 @@ extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, in
   const int dkp = (Dk + 31) & ~31;
   int LD = dkp + 16;
   while ((LD & 63) != 16) LD += 8;
-  const size_t smem = (size_t)LM_KEYS * LD * sizeof(bf16_t);
+  const size_t smem = (size_t)2 * LM_KEYS * LD * sizeof(bf16_t);  // two buffers that take turns
   // `split` > 0: every tile is a single row (the caller's promise), whose keys are cut into absolute ranges of `split`
   // keys over n_z workgroups; `part` holds rows x H x n_z x (R + 4) floats
   if (split > 0 && ((split & 63) || n_z < 1 || n_z > 65535 || !part)) JLLM_FAIL("latent_attention: ranges of %d keys over %d workgroups", split, n_z);

@@ -8,9 +8,10 @@
 #include "mfma.h"
 
 #define MM_WAVES 4
-#define MM_ROWS 16
 
-template <bool GATED>
+// RB: 16-row blocks of a tile (tiles of 16 rows for steps with few rows per expert, of 64 where experts get many: a
+// weight fragment then meets four activation fragments)
+template <bool GATED, int RB>
 __global__ __launch_bounds__(MM_WAVES * 64) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     void* __restrict__ out, int out_dtype, int ldo, int N, int K, const int* __restrict__ sorted,
@@ -24,43 +25,63 @@ __global__ __launch_bounds__(MM_WAVES * 64) void moe_gemm_mfma_kernel(
   constexpr int NB = GATED ? 2 : 4;  // 16-output blocks per wave
   const int n0 = (blockIdx.x * MM_WAVES + wave) * (16 * NB);
   if (n0 >= N) return;
-  const int place = first + min(sub, rows - 1);
-  const int asg = sorted[place];
-  const bf16_t* xrow = A + (size_t)(in_map ? asg / top : place) * lda + 8 * q4;
+  int place[RB], asg[RB];
+  const bf16_t* xrow[RB];
+#pragma unroll
+  for (int rb = 0; rb < RB; ++rb) {
+    place[rb] = first + min(16 * rb + sub, rows - 1);
+    asg[rb] = sorted[place[rb]];
+    xrow[rb] = A + (size_t)(in_map ? asg[rb] / top : place[rb]) * lda + 8 * q4;
+  }
   const bf16_t* w = W + (size_t)e * N * K + 8 * q4;
   const bf16_t* w2 = GATED ? W2 + (size_t)e * N * K + 8 * q4 : nullptr;
-  floatx4 acc[NB], acc2[NB];
+  floatx4 acc[RB][NB], acc2[RB][NB];
 #pragma unroll
-  for (int b = 0; b < NB; ++b) acc[b] = acc2[b] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+    for (int b = 0; b < NB; ++b) acc[rb][b] = acc2[rb][b] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool in_k = k0 + 8 * q4 < K;
-    const u32x4 xf = in_k ? *(const u32x4*)(xrow + k0) : u32x4{0u, 0u, 0u, 0u};
+    u32x4 xf[RB], wf[NB], uf[NB];
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb) xf[rb] = in_k ? *(const u32x4*)(xrow[rb] + k0) : u32x4{0u, 0u, 0u, 0u};
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
       const int n = n0 + 16 * b + sub;
       const bool ok = in_k && n < N;
-      acc[b] = mfma16(ok ? *(const u32x4*)(w + (size_t)n * K + k0) : u32x4{0u, 0u, 0u, 0u}, xf, acc[b]);
-      if (GATED) acc2[b] = mfma16(ok ? *(const u32x4*)(w2 + (size_t)n * K + k0) : u32x4{0u, 0u, 0u, 0u}, xf, acc2[b]);
+      wf[b] = ok ? *(const u32x4*)(w + (size_t)n * K + k0) : u32x4{0u, 0u, 0u, 0u};
+      if (GATED) uf[b] = ok ? *(const u32x4*)(w2 + (size_t)n * K + k0) : u32x4{0u, 0u, 0u, 0u};
     }
+#pragma unroll
+    for (int rb = 0; rb < RB; ++rb)
+#pragma unroll
+      for (int b = 0; b < NB; ++b) {
+        acc[rb][b] = mfma16(wf[b], xf[rb], acc[rb][b]);
+        if (GATED) acc2[rb][b] = mfma16(uf[b], xf[rb], acc2[rb][b]);
+      }
   }
-  if (sub >= rows) return;
-  const size_t orow = out_map == 0 ? (size_t)place : out_map == 1 ? (size_t)asg : (size_t)(asg / top);
 #pragma unroll
-  for (int b = 0; b < NB; ++b) {
-    const int n = n0 + 16 * b + 4 * q4;
-    if (n >= N) continue;
-    float v[4];
+  for (int rb = 0; rb < RB; ++rb) {
+    if (16 * rb + sub >= rows) continue;
+    const size_t orow = out_map == 0 ? (size_t)place[rb] : out_map == 1 ? (size_t)asg[rb] : (size_t)(asg[rb] / top);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) v[i] = GATED ? gated<true>(acc[b][i], acc2[b][i], gs) : acc[b][i];
-    const size_t o = orow * ldo + n;
-    if (out_map == 2) {
-      floatx4* dst = (floatx4*)((float*)out + o);
-      const floatx4 cur = *dst;
-      *dst = floatx4{cur[0] + weight * v[0], cur[1] + weight * v[1], cur[2] + weight * v[2], cur[3] + weight * v[3]};
-    } else if (out_dtype == JLLM_BF16) {
-      *(u32x2*)((bf16_t*)out + o) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
-    } else {
-      *(floatx4*)((float*)out + o) = floatx4{v[0], v[1], v[2], v[3]};
+    for (int b = 0; b < NB; ++b) {
+      const int n = n0 + 16 * b + 4 * q4;
+      if (n >= N) continue;
+      float v[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) v[i] = GATED ? gated<true>(acc[rb][b][i], acc2[rb][b][i], gs) : acc[rb][b][i];
+      const size_t o = orow * ldo + n;
+      if (out_map == 2) {
+        floatx4* dst = (floatx4*)((float*)out + o);
+        const floatx4 cur = *dst;
+        *dst = floatx4{cur[0] + weight * v[0], cur[1] + weight * v[1], cur[2] + weight * v[2], cur[3] + weight * v[3]};
+      } else if (out_dtype == JLLM_BF16) {
+        *(u32x2*)((bf16_t*)out + o) = u32x2{pack_bf16(v[0], v[1]), pack_bf16(v[2], v[3])};
+      } else {
+        *(floatx4*)((float*)out + o) = floatx4{v[0], v[1], v[2], v[3]};
+      }
     }
   }
 }
@@ -73,7 +94,7 @@ extern "C" int jllm_moe_gemm_bf16(const void* A, int a_dtype, int lda, const voi
   if (max_tiles <= 0) return 0;
   if (a_dtype != JLLM_BF16 || w_dtype != JLLM_BF16) return 1;
   if (N <= 0 || K <= 0 || lda < K || ldo < N) JLLM_FAIL("moe_gemm: N %d K %d lda %d ldo %d", N, K, lda, ldo);
-  if (tile_rows != MM_ROWS) JLLM_FAIL("moe_gemm: this kernel takes tiles of %d rows, the route made %d", MM_ROWS, tile_rows);
+  if (tile_rows != 16 && tile_rows != 64) JLLM_FAIL("moe_gemm: this kernel takes tiles of 16 or 64 rows, the route made %d", tile_rows);
   JLLM_TAKE_GATE("moe_gemm", epilogue, gate_limit, gs);
   if ((epilogue != 0 && epilogue != 2) || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("moe_gemm: epilogue %d", epilogue);
   if (in_map < 0 || in_map > 1 || out_map < 0 || out_map > 2) JLLM_FAIL("moe_gemm: maps %d / %d", in_map, out_map);
@@ -85,12 +106,18 @@ extern "C" int jllm_moe_gemm_bf16(const void* A, int a_dtype, int lda, const voi
   if (((uintptr_t)out & need) || (ldo & 3)) return 1;
   const int per_group = MM_WAVES * 16 * (W2 ? 2 : 4);
   dim3 grid((N + per_group - 1) / per_group, max_tiles);
-  if (W2)
-    moe_gemm_mfma_kernel<true><<<grid, MM_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, out,
-                                                                   out_dtype, ldo, N, K, sorted, tiles, top, in_map, out_map, weight, gs);
+#define MM_LAUNCH(GATED, RB)                                                                                                    \
+  moe_gemm_mfma_kernel<GATED, RB><<<grid, MM_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, out, \
+                                                                      out_dtype, ldo, N, K, sorted, tiles, top, in_map, out_map, weight, gs)
+  if (W2 && tile_rows == 64)
+    MM_LAUNCH(true, 4);
+  else if (W2)
+    MM_LAUNCH(true, 1);
+  else if (tile_rows == 64)
+    MM_LAUNCH(false, 4);
   else
-    moe_gemm_mfma_kernel<false><<<grid, MM_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, out, out_dtype,
-                                                                    ldo, N, K, sorted, tiles, top, in_map, out_map, weight, gs);
+    MM_LAUNCH(false, 1);
+#undef MM_LAUNCH
   JLLM_CHECK_LAUNCH("moe_gemm_bf16");
   return 0;
 }

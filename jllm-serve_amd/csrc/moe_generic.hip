@@ -94,9 +94,10 @@ __global__ __launch_bounds__(256) void moe_gemm_generic_kernel(
     int out_dtype, int ldo, int N, int K, const int* __restrict__ sorted, const int* __restrict__ tiles, int top,
     int in_map, int out_map, float weight, GateSpec gs) {
   const int tile = blockIdx.y;
-  const int rows = tiles[3 * tile + 2];
-  if (rows == 0) return;
-  const int e = tiles[3 * tile], first = tiles[3 * tile + 1];
+  // a tile of more than MG_ROWS rows is taken MG_ROWS at a time, over gridDim.z
+  const int rows = min(MG_ROWS, tiles[3 * tile + 2] - MG_ROWS * (int)blockIdx.z);
+  if (rows <= 0) return;
+  const int e = tiles[3 * tile], first = tiles[3 * tile + 1] + MG_ROWS * (int)blockIdx.z;
   __shared__ float As[MG_K][MG_ROWS + 1];
   __shared__ float Ws[MG_K][MG_COLS + 4];
   __shared__ float Us[GATED ? MG_K : 1][MG_COLS + 4];
@@ -160,13 +161,13 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
                                      int epilogue, float gate_limit, hipStream_t stream) {
   if (max_tiles <= 0) return 0;
   if (N <= 0 || K <= 0 || lda < K || ldo < N) JLLM_FAIL("moe_gemm: N %d K %d lda %d ldo %d", N, K, lda, ldo);
-  if (tile_rows != MG_ROWS) JLLM_FAIL("moe_gemm: this kernel takes tiles of %d rows, the route made %d", MG_ROWS, tile_rows);
+  if (tile_rows <= 0 || tile_rows % MG_ROWS) JLLM_FAIL("moe_gemm: this kernel takes tiles of multiples of %d rows, the route made %d", MG_ROWS, tile_rows);
   if (max_tiles > 65535) JLLM_FAIL("moe_gemm: %d tiles are too many for one launch", max_tiles);
   JLLM_TAKE_GATE("moe_gemm", epilogue, gate_limit, gs);
   if ((epilogue != 0 && epilogue != 2) || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("moe_gemm: epilogue %d", epilogue);
   if (in_map < 0 || in_map > 1 || out_map < 0 || out_map > 2) JLLM_FAIL("moe_gemm: maps %d / %d", in_map, out_map);
   if (out_map == 2 && (top != 1 || out_dtype != JLLM_F32)) JLLM_FAIL("moe_gemm: adding into the token's row needs top = 1 and fp32 rows");
-  dim3 grid((N + MG_COLS - 1) / MG_COLS, max_tiles);
+  dim3 grid((N + MG_COLS - 1) / MG_COLS, max_tiles, tile_rows / MG_ROWS);
   JLLM_DISPATCH_1(a_dtype, TA, {
     JLLM_DISPATCH_1(w_dtype, TW, {
       if (W2)

@@ -986,13 +986,14 @@ def _latent_split(rows: int, heads: int, window: int, max_ctx: int):
 
 # ------------------------------------------------------------------------------------------------ table-routed experts
 
-MOE_TILE_ROWS = 16     # rows of one expert that a workgroup of the grouped products takes
+MOE_TILE_ROWS = 16     # rows of one expert that a workgroup of the grouped products takes ...
+MOE_TILE_ROWS_MANY = 64  # ... and where the experts get this many rows each on average (portions of prompts)
 
 
 def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
     """Groups the assignments (row t, k-th expert of its token) by expert, on the device: returns (sorted [T * top]
     int32: the assignments t * top + k expert by expert; tiles [max_tiles, 3] int32: expert, first place in sorted,
-    rows (0 = unused); max_tiles)."""
+    rows (0 = unused); max_tiles; rows a tile holds at most: 16, or 64 in steps that give the experts many rows)."""
     _dev(token_ids, table)
     T = token_ids.numel()
     _i32(token_ids, T, "token ids")
@@ -1000,12 +1001,13 @@ def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
         raise KernelError("the routing table must be a contiguous int32 [vocab, top] tensor")
     top = table.shape[1]
     A = T * top
-    max_tiles = max(1, min(A, A // MOE_TILE_ROWS + experts))
+    tile_rows = MOE_TILE_ROWS_MANY if A >= MOE_TILE_ROWS_MANY * experts else MOE_TILE_ROWS
+    max_tiles = max(1, min(A, A // tile_rows + experts))
     sorted_ = torch.empty((max(A, 1),), dtype=torch.int32, device=table.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=table.device)
-    _call("jllm_moe_route", _ptr(token_ids), _ptr(table), T, top, experts, MOE_TILE_ROWS, max_tiles, _ptr(sorted_), _ptr(tiles),
+    _call("jllm_moe_route", _ptr(token_ids), _ptr(table), T, top, experts, tile_rows, max_tiles, _ptr(sorted_), _ptr(tiles),
           _stream())
-    return sorted_, tiles, max_tiles
+    return sorted_, tiles, max_tiles, tile_rows
 
 
 def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optional[torch.Tensor] = None,
@@ -1015,7 +1017,7 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optiona
     expert's weights ``w[e]`` ([experts, N, K]); with ``w2`` the gate function is applied to the two sums. ``in_map``
     0 / 1: a tile's input rows are its places in the sorted order / its assignments' token rows; ``out_map`` 0 / 1 / 2:
     output rows by place / by assignment / added, times ``weight``, into the fp32 row of the token (top = 1)."""
-    sorted_, tiles, max_tiles = routing
+    sorted_, tiles, max_tiles, tile_rows = routing
     _dev(a, w, w2, out)
     _rows2d(a, "moe input")
     _rows2d(out, "moe output")
@@ -1026,7 +1028,7 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optiona
         raise KernelError(f"moe_gemm: rows of {a.shape[1]} -> {out.shape[1]} with weights {tuple(w.shape)}")
     epilogue = (EPI_GATED | (int(gate) << 8)) if w2 is not None else EPI_STORE
     head = (_ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(out), _code(out.dtype),
-            out.stride(0), N, K, _ptr(sorted_), _ptr(tiles), max_tiles, MOE_TILE_ROWS, int(top), int(in_map), int(out_map),
+            out.stride(0), N, K, _ptr(sorted_), _ptr(tiles), max_tiles, tile_rows, int(top), int(in_map), int(out_map),
             float(weight), epilogue, float(gate_limit), _stream())
     if not exact and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _try("jllm_moe_gemm_bf16", *head):
         return out

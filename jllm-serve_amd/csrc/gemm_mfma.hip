@@ -28,7 +28,8 @@ template <bool GATED, int WGM, int WGN, int FM, int FN, bool DEEP>
 __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
     const void* __restrict__ bias, int bias_dtype, void* __restrict__ out, int out_dtype, int ldo, int M, int N, int K,
-    int epilogue, GateSpec gs, float* __restrict__ partial) {
+    int epilogue, GateSpec gs, float* __restrict__ partial, const int* __restrict__ groups, const int* __restrict__ row_map,
+    int row_div) {
   static_assert(FN == 2, "a wave's columns are two 32-wide accumulators (gate and up with the gated epilogue)");
   constexpr int NT = WGM * WGN * 64;
   constexpr int TBM = WGM * FM * 32, TBN = WGN * FN * 32;
@@ -40,14 +41,30 @@ __global__ __launch_bounds__(WGM* WGN * 64) void gemm_mfma_kernel(
   const int tid = threadIdx.x;
   const int wave = tid >> 6, lane = tid & 63;
   const int wm = wave / WGN, wn = wave % WGN;
-  const int m0 = blockIdx.y * TBM;
+  // Grouped form (`groups`: (group, first row, rows) per blockIdx.y, rows = 0 for an unused entry): the workgroup's rows
+  // are first .. first + rows - 1, its weights those of its group ([groups][N][K]); with `row_map` input row i is row
+  // row_map[i] / row_div of A (rows gathered by an index list), the output rows stay i.
+  int m0 = blockIdx.y * TBM;
+  if (groups) {
+    const int g_rows = groups[3 * blockIdx.y + 2];
+    if (g_rows == 0) return;
+    m0 = groups[3 * blockIdx.y + 1];
+    M = m0 + g_rows;
+    const size_t at = (size_t)groups[3 * blockIdx.y] * N * K;
+    W += at;
+    if (GATED) W2 += at;
+  }
   const int n0 = blockIdx.x * (GATED ? TBN / 2 : TBN);  // output columns covered by this workgroup start here
   // global -> register staging: piece c = tid + NT j: row c / TPCS, 16 bytes number c % TPCS
   const int lrow = tid / TPCS, lpc = tid % TPCS;
   const bf16_t* aptr[PA];
   const bf16_t* bptr[PB];
 #pragma unroll
-  for (int j = 0; j < PA; ++j) aptr[j] = A + (size_t)min(m0 + lrow + TRSTEP * j, M - 1) * lda + lpc * 8;
+  for (int j = 0; j < PA; ++j) {
+    int row = min(m0 + lrow + TRSTEP * j, M - 1);
+    if (row_map) row = row_map[row] / row_div;
+    aptr[j] = A + (size_t)row * lda + lpc * 8;
+  }
 #pragma unroll
   for (int j = 0; j < PB; ++j) {
     const int r = lrow + TRSTEP * j;
@@ -248,10 +265,10 @@ static int launch_tiled(const void* A, int lda, const void* W, const void* W2, c
   }
   if (W2)
     gemm_mfma_kernel<true, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, nullptr, nullptr, 1);
   else
     gemm_mfma_kernel<false, WGM, WGN, FM, FN, DEEP><<<grid, WGM * WGN * 64, smem, stream>>>(
-        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial);
+        (const bf16_t*)A, lda, (const bf16_t*)W, nullptr, bias, bias_dtype, out, out_dtype, ldo, M, N, K, epilogue, gs, partial, nullptr, nullptr, 1);
   return 0;
 }
 
@@ -290,5 +307,41 @@ extern "C" int jllm_gemm_mfma_bf16(const void* A, int lda, const void* W, const 
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("gemm_mfma");
   if (splits > 1) return jllm_splitk_reduce(partial, splits, bias, bias_dtype, out, out_dtype, ldo, M, N, epilogue, stream);
+  return 0;
+}
+
+// The grouped form of the small tile: `tiles` holds (group, first row, rows <= 128) per entry (rows = 0: unused), the
+// weights are [groups][N][K] (and W2 likewise for the gated epilogue), row i of the input is A[row_map[i] / row_div]
+// when `row_map` is given, and output row i is row i of `out`. K whole, epilogues store and gated.
+// returns 0 when it ran, 1 when the shape is not one it takes, -1 on errors
+extern "C" int jllm_gemm_mfma_grouped_bf16(const void* A, int lda, const void* W, const void* W2, void* out, int out_dtype,
+                                           int ldo, int M, int N, int K, int epilogue, float gate_limit, const int* tiles,
+                                           int max_tiles, int tile_rows, const int* row_map, int row_div,
+                                           hipStream_t stream) {
+  if (max_tiles <= 0 || M <= 0) return 0;
+  if ((K & 63) || K <= 0 || N <= 0 || (lda & 7) || max_tiles > 65535) return 1;
+  if (((uintptr_t)A & 15) || ((uintptr_t)W & 15) || (W2 && ((uintptr_t)W2 & 15))) return 1;
+  JLLM_TAKE_GATE("gemm_mfma_grouped", epilogue, gate_limit, gs);
+  if ((epilogue != 0 && epilogue != 2) || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("gemm_mfma_grouped: epilogue %d", epilogue);
+  constexpr int TBM = 128, TBN = 128;
+  if (tile_rows != TBM) JLLM_FAIL("gemm_mfma_grouped: tiles of %d rows, this kernel takes %d", tile_rows, TBM);
+  if (ldo < N || row_div < 1) JLLM_FAIL("gemm_mfma_grouped: ldo %d < N %d", ldo, N);
+  const int cols = W2 ? TBN / 2 : TBN;
+  dim3 grid((N + cols - 1) / cols, max_tiles, 1);
+  const size_t smem = (size_t)2 * (TBM + TBN) * TLD * sizeof(bf16_t);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t e1 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<true, 2, 2, 2, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    hipError_t e2 = hipFuncSetAttribute((const void*)gemm_mfma_kernel<false, 2, 2, 2, 2, false>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    if (e1 != hipSuccess || e2 != hipSuccess) JLLM_FAIL("gemm_mfma_grouped: cannot reserve %zu bytes of LDS", smem);
+    configured = true;
+  }
+  if (W2)
+    gemm_mfma_kernel<true, 2, 2, 2, 2, false><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, nullptr, 0, out,
+                                                                           out_dtype, ldo, M, N, K, epilogue, gs, nullptr, tiles, row_map, row_div);
+  else
+    gemm_mfma_kernel<false, 2, 2, 2, 2, false><<<grid, 256, smem, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, nullptr, nullptr, 0, out, out_dtype,
+                                                                            ldo, M, N, K, epilogue, gs, nullptr, tiles, row_map, row_div);
+  JLLM_CHECK_LAUNCH("gemm_mfma_grouped");
   return 0;
 }

@@ -84,38 +84,26 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
 #pragma unroll
   for (int j = 0; j < RT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m1 = -INFINITY, l1 = 0.f;
-  const int chunks = dks * 4;  // 16-byte pieces of a staged row (zero beyond Dk)
   // A block of 64 keys goes global -> registers -> LDS. All of a thread's pieces are requested together (first their
   // table entries, then the rows: two latencies a block, not two per piece), and the next block's are requested before
   // this block is multiplied, into the other of two LDS buffers: one barrier per block.
-  constexpr int CPT = (LM_KEYS * DKS * 4 + LM_WAVES * 64 - 1) / (LM_WAVES * 64);
+  // four threads to a key row (256 threads, 64 rows): a thread's pieces are 16 bytes at (tid % 4) * 16 + 64 i of its row:
+  // one table entry and one address per block
+  constexpr int CPT = DKS;
+  static_assert(LM_WAVES * 64 == 4 * LM_KEYS, "four threads stage a key row");
   uint4 staged[CPT];
+  const int srow = threadIdx.x >> 2, scol = (threadIdx.x & 3) * 8;
   auto fetch = [&](int blk) {
-    const int c0 = blk * LM_KEYS;
-    int page[CPT];
+    const int key = min(max(blk * LM_KEYS + srow, kb), ke);  // a key outside the range is masked below and reads one inside it
+    const bf16_t* src = cache + ((((size_t)tbl[key >> psh]) << psh) + (key & (page_size - 1))) * Dk + scol;
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int idx = threadIdx.x + LM_WAVES * 64 * i;
-      const int key = min(max(c0 + idx / chunks, kb), ke);  // a key outside the range is masked below and reads one inside it
-      page[i] = tbl[key >> psh];
-    }
-#pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int idx = threadIdx.x + LM_WAVES * 64 * i;
-      const int r = idx / chunks, c = idx - r * chunks;
-      const int key = min(max(c0 + r, kb), ke);
-      staged[i] = uint4{0u, 0u, 0u, 0u};
-      if (idx < LM_KEYS * chunks && 8 * c < Dk)
-        staged[i] = *(const uint4*)(cache + ((((size_t)page[i]) << psh) + (key & (page_size - 1))) * Dk + 8 * c);
-    }
+    for (int i = 0; i < CPT; ++i) staged[i] = (i < dks && scol + 32 * i < Dk) ? *(const uint4*)(src + 32 * i) : uint4{0u, 0u, 0u, 0u};
   };
   auto put = [&](bf16_t* buf) {
+    bf16_t* dst = buf + srow * LD + scol;
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) {
-      const int idx = threadIdx.x + LM_WAVES * 64 * i;
-      const int r = idx / chunks, c = idx - r * chunks;
-      if (idx < LM_KEYS * chunks) *(uint4*)(buf + r * LD + 8 * c) = staged[i];
-    }
+    for (int i = 0; i < CPT; ++i)
+      if (i < dks) *(uint4*)(dst + 32 * i) = staged[i];
   };
   const int blk_last = ke >> 6;
   int cur = 0;

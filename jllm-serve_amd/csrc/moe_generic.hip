@@ -8,7 +8,8 @@
 //                 [N, K]. The first product gathers its input rows by token (assignment / top), applies the gate
 //                 function to the two sums and writes hidden rows in the order of `sorted`; the second reads those
 //                 and writes fp32 rows by assignment, or, with top = 1, adds them straight into the residual rows
-//   moe_combine   residual[t] += weight * sum_k y[t * top + k], k ascending
+//   moe_combine   residual[t] += weight * sum_k y[t * top + k], k ascending (or y[place_of[t * top + k]] where the second
+//                 product wrote its rows in the order of `sorted`)
 //
 // The order of `sorted` within an expert comes from LDS atomics and may differ between runs; no result depends on it
 // (every output is one accumulator over ascending k of its own row and weight row). This file is the fp32 path
@@ -19,7 +20,8 @@
 
 __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int* __restrict__ tokens, const int* __restrict__ table,
                                                                      int T, int top, int E, int tile_rows, int max_tiles,
-                                                                     int* __restrict__ sorted, int* __restrict__ tiles) {
+                                                                     int* __restrict__ sorted, int* __restrict__ tiles,
+                                                                     int* __restrict__ place_of) {
   extern __shared__ int sh[];
   int* count = sh;           // [E]
   int* start = sh + E;       // [E + 1]
@@ -52,7 +54,9 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int*
   __syncthreads();
   for (int a = threadIdx.x; a < A; a += MOE_ROUTE_THREADS) {
     const int e = table[(size_t)tokens[a / top] * top + a % top];
-    sorted[start[e] + atomicAdd(&cursor[e], 1)] = a;
+    const int place = start[e] + atomicAdd(&cursor[e], 1);
+    sorted[place] = a;
+    if (place_of) place_of[a] = place;
   }
   for (int e = threadIdx.x; e < E; e += MOE_ROUTE_THREADS) {
     const int c = count[e];
@@ -67,7 +71,7 @@ __global__ __launch_bounds__(MOE_ROUTE_THREADS) void moe_route_kernel(const int*
 }
 
 extern "C" int jllm_moe_route(const int* tokens, const int* table, int T, int top, int E, int tile_rows, int max_tiles,
-                              int* sorted, int* tiles, hipStream_t stream) {
+                              int* sorted, int* tiles, int* place_of, hipStream_t stream) {
   if (T <= 0) return 0;
   if (top <= 0 || E <= 0 || top > E || tile_rows <= 0) JLLM_FAIL("moe_route: top %d of %d experts, tiles of %d rows", top, E, tile_rows);
   const long A = (long)T * top;
@@ -75,7 +79,7 @@ extern "C" int jllm_moe_route(const int* tokens, const int* table, int T, int to
   if (max_tiles < need) JLLM_FAIL("moe_route: room for %d tiles, %ld may be needed", max_tiles, need);
   const size_t smem = (size_t)(4 * E + 2) * sizeof(int);
   if (smem > 64 * 1024) JLLM_FAIL("moe_route: %d experts are more than this kernel's LDS holds", E);
-  moe_route_kernel<<<1, MOE_ROUTE_THREADS, smem, stream>>>(tokens, table, T, top, E, tile_rows, max_tiles, sorted, tiles);
+  moe_route_kernel<<<1, MOE_ROUTE_THREADS, smem, stream>>>(tokens, table, T, top, E, tile_rows, max_tiles, sorted, tiles, place_of);
   JLLM_CHECK_LAUNCH("moe_route");
   return 0;
 }
@@ -184,19 +188,23 @@ extern "C" int jllm_moe_gemm_generic(const void* A, int a_dtype, int lda, const 
 
 // ---------------------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ residual, int width,
-                                                         int top, float weight) {
+                                                         int top, float weight, const int* __restrict__ place_of) {
   const int t = blockIdx.x;
   for (int i = threadIdx.x; i < width; i += 256) {
     float s = 0.f;
-    for (int k = 0; k < top; ++k) s += y[((size_t)t * top + k) * width + i];
+    for (int k = 0; k < top; ++k) {
+      const size_t row = place_of ? (size_t)place_of[t * top + k] : (size_t)t * top + k;
+      s += y[row * width + i];
+    }
     residual[(size_t)t * width + i] += weight * s;
   }
 }
 
-extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, hipStream_t stream) {
+extern "C" int jllm_moe_combine(const float* y, float* residual, int T, int width, int top, float weight, const int* place_of,
+                                hipStream_t stream) {
   if (T <= 0) return 0;
   if (width <= 0 || top <= 0) JLLM_FAIL("moe_combine: width %d top %d", width, top);
-  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight);
+  moe_combine_kernel<<<T, 256, 0, stream>>>(y, residual, width, top, weight, place_of);
   JLLM_CHECK_LAUNCH("moe_combine");
   return 0;
 }

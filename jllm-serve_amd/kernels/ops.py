@@ -71,9 +71,9 @@ def _declare(lib) -> None:
         "jllm_latent_prepare": [_P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _P, _P, _P, _I, _P, _P],
         "jllm_latent_heads_generic": [_P, _I, _I, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
         "jllm_latent_attention_generic": [_P, _I, _P, _I, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _P],
-        "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P],
+        "jllm_moe_route": [_P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P],
         "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
-        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P],
+        "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
     }
     for name, args in sig.items():
@@ -106,6 +106,7 @@ _OPTIONAL_SIGS = {
     "jllm_prefill_attention_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
+    "jllm_gemm_mfma_grouped_bf16": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _I, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -986,14 +987,28 @@ def _latent_split(rows: int, heads: int, window: int, max_ctx: int):
 
 # ------------------------------------------------------------------------------------------------ table-routed experts
 
-MOE_TILE_ROWS = 16     # rows of one expert that a workgroup of the grouped products takes ...
-MOE_TILE_ROWS_MANY = 64  # ... and where the experts get this many rows each on average (portions of prompts)
+MOE_TILE_ROWS = 16      # rows of one expert that a workgroup of the grouped products takes in steps of few rows ...
+MOE_TILE_ROWS_MANY = 128  # ... and where the experts get many rows each (portions of prompts): the tiled product's tile
 
 
-def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
-    """Groups the assignments (row t, k-th expert of its token) by expert, on the device: returns (sorted [T * top]
-    int32: the assignments t * top + k expert by expert; tiles [max_tiles, 3] int32: expert, first place in sorted,
-    rows (0 = unused); max_tiles; rows a tile holds at most: 16, or 64 in steps that give the experts many rows)."""
+class MoeRouting:
+    """What ``moe_route`` made of a step: ``sorted`` [T * top] (the assignments t * top + k expert by expert), ``tiles``
+    [max_tiles, 3] (expert, first place in sorted, rows; 0 rows = unused), ``place_of`` [T * top] (where each
+    assignment lies in sorted) and the rows a tile holds at most."""
+
+    def __init__(self, sorted_, tiles, place_of, max_tiles, tile_rows, top):
+        self.sorted, self.tiles, self.place_of = sorted_, tiles, place_of
+        self.max_tiles, self.tile_rows, self.top = max_tiles, tile_rows, top
+
+    @property
+    def many(self) -> bool:
+        return self.tile_rows == MOE_TILE_ROWS_MANY
+
+
+def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int, many_ok: bool = False) -> MoeRouting:
+    """Groups the assignments (row t, k-th expert of its token) by expert, on the device. ``many_ok``: the caller's
+    products can go through the tiled matrix-core kernel (bf16, K a multiple of 64): steps that give the experts 64 rows
+    or more each on average are then cut into tiles of 128 rows, all others into tiles of 16."""
     _dev(token_ids, table)
     T = token_ids.numel()
     _i32(token_ids, T, "token ids")
@@ -1001,35 +1016,45 @@ def moe_route(token_ids: torch.Tensor, table: torch.Tensor, experts: int):
         raise KernelError("the routing table must be a contiguous int32 [vocab, top] tensor")
     top = table.shape[1]
     A = T * top
-    tile_rows = MOE_TILE_ROWS_MANY if A >= MOE_TILE_ROWS_MANY * experts else MOE_TILE_ROWS
+    tile_rows = MOE_TILE_ROWS_MANY if many_ok and A >= 64 * experts else MOE_TILE_ROWS
     max_tiles = max(1, min(A, A // tile_rows + experts))
     sorted_ = torch.empty((max(A, 1),), dtype=torch.int32, device=table.device)
+    place_of = torch.empty((max(A, 1),), dtype=torch.int32, device=table.device)
     tiles = torch.empty((max_tiles, 3), dtype=torch.int32, device=table.device)
     _call("jllm_moe_route", _ptr(token_ids), _ptr(table), T, top, experts, tile_rows, max_tiles, _ptr(sorted_), _ptr(tiles),
-          _stream())
-    return sorted_, tiles, max_tiles, tile_rows
+          _ptr(place_of), _stream())
+    return MoeRouting(sorted_, tiles, place_of, max_tiles, tile_rows, top)
 
 
-def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optional[torch.Tensor] = None,
+def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing: MoeRouting, *, w2: Optional[torch.Tensor] = None,
              out: torch.Tensor, in_map: int, out_map: int, weight: float = 1.0, gate: int = 0, gate_limit: float = 0.0,
              exact: bool = False) -> torch.Tensor:
     """The grouped product of a routed feed-forward: every tile of ``routing`` multiplies its rows of ``a`` with its
     expert's weights ``w[e]`` ([experts, N, K]); with ``w2`` the gate function is applied to the two sums. ``in_map``
     0 / 1: a tile's input rows are its places in the sorted order / its assignments' token rows; ``out_map`` 0 / 1 / 2:
-    output rows by place / by assignment / added, times ``weight``, into the fp32 row of the token (top = 1)."""
-    sorted_, tiles, max_tiles, tile_rows = routing
+    output rows by place / by assignment / added, times ``weight``, into the fp32 row of the token (top = 1). With
+    tiles of many rows (``routing.many``) the tiled matrix-core kernel takes the product; its output rows go by place."""
     _dev(a, w, w2, out)
     _rows2d(a, "moe input")
     _rows2d(out, "moe output")
     if w.dim() != 3 or not w.is_contiguous() or (w2 is not None and (w2.shape != w.shape or w2.dtype != w.dtype or not w2.is_contiguous())):
         raise KernelError("moe weights must be contiguous [experts, N, K] tensors of one shape and type")
     _, N, K = w.shape
+    top = routing.top
     if a.shape[1] != K or out.shape[1] != N:
         raise KernelError(f"moe_gemm: rows of {a.shape[1]} -> {out.shape[1]} with weights {tuple(w.shape)}")
     epilogue = (EPI_GATED | (int(gate) << 8)) if w2 is not None else EPI_STORE
+    if routing.many:
+        if out_map != 0 or exact or a.dtype != torch.bfloat16 or w.dtype != torch.bfloat16:
+            raise KernelError("moe_gemm: tiles of many rows go through the bf16 tiled kernel and write their rows by place")
+        if not _try("jllm_gemm_mfma_grouped_bf16", _ptr(a), a.stride(0), _ptr(w), _ptr(w2), _ptr(out), _code(out.dtype),
+                    out.stride(0), routing.sorted.numel(), N, K, epilogue, float(gate_limit), _ptr(routing.tiles),
+                    routing.max_tiles, routing.tile_rows, _ptr(routing.sorted) if in_map else None, int(top), _stream()):
+            raise KernelError(f"moe_gemm: the tiled kernel does not take N {N}, K {K} (K must be a multiple of 64)")
+        return out
     head = (_ptr(a), _code(a.dtype), a.stride(0), _ptr(w), _ptr(w2), _code(w.dtype), _ptr(out), _code(out.dtype),
-            out.stride(0), N, K, _ptr(sorted_), _ptr(tiles), max_tiles, tile_rows, int(top), int(in_map), int(out_map),
-            float(weight), epilogue, float(gate_limit), _stream())
+            out.stride(0), N, K, _ptr(routing.sorted), _ptr(routing.tiles), routing.max_tiles, routing.tile_rows, int(top),
+            int(in_map), int(out_map), float(weight), epilogue, float(gate_limit), _stream())
     if not exact and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and _try("jllm_moe_gemm_bf16", *head):
         return out
     if not exact:
@@ -1038,14 +1063,16 @@ def moe_gemm(a: torch.Tensor, w: torch.Tensor, routing, top: int, *, w2: Optiona
     return out
 
 
-def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float) -> None:
-    """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending)."""
-    _dev(y, residual)
+def moe_combine(y: torch.Tensor, residual: torch.Tensor, top: int, weight: float, place_of: Optional[torch.Tensor] = None) -> None:
+    """residual[t] += weight * sum_k y[t * top + k] (fp32 both; k ascending); with ``place_of`` the k-th row of t is
+    y[place_of[t * top + k]]."""
+    _dev(y, residual, place_of)
     T, width = residual.shape
     if y.dtype != torch.float32 or residual.dtype != torch.float32 or not y.is_contiguous() or not residual.is_contiguous() \
             or y.shape != (T * top, width):
         raise KernelError("moe_combine takes contiguous fp32 [T * top, width] rows and the fp32 residual [T, width]")
-    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _stream())
+    _i32(place_of, T * top, "places")
+    _call("jllm_moe_combine", _ptr(y), _ptr(residual), T, width, int(top), float(weight), _ptr(place_of), _stream())
 
 
 def argmax(logits: torch.Tensor) -> torch.Tensor:

@@ -7,7 +7,7 @@ the spec has one, is a dense gated feed-forward that runs for every row.
 The routing happens on the device from the step's token ids (``ops.moe_route``), the experts' products are grouped
 launches over tiles of rows of one expert (``ops.moe_gemm``): gate/up gathers the rows by token and writes hidden rows
 in expert order; down writes per assignment (summed into the residual by ``ops.moe_combine``) or, with top = 1, adds
-into the residual itself. Nothing waits for the GPU, so a decode step with this feed-forward can be captured.
+into the residual itself. Steps with many rows per expert use tiles of 128 rows through the tiled matrix-core product. Nothing waits for the GPU, so a decode step with this feed-forward can be captured.
 """
 from __future__ import annotations
 
@@ -68,16 +68,23 @@ class TableMoe(Part):
         T = xb.shape[0]
         if self.shared is not None:
             self.shared.forward(xb, residual, step)
-        routing = ops.moe_route(step.token_ids, self.table, s.experts)
+        # portions of prompts (many rows per expert) go through the tiled matrix-core product, whose K steps are 64 wide
+        many_ok = not exact and self.build.dtype == torch.bfloat16 and self.w_gate.dtype == torch.bfloat16 \
+            and residual.shape[1] % 64 == 0 and s.hidden % 64 == 0
+        routing = ops.moe_route(step.token_ids, self.table, s.experts, many_ok=many_ok)
         A = T * s.top
         hidden = torch.empty((A, s.hidden), dtype=self.build.dtype, device=xb.device)
-        ops.moe_gemm(xb, self.w_gate, routing, s.top, w2=self.w_up, out=hidden, in_map=1, out_map=0, gate=self.gate,
+        ops.moe_gemm(xb, self.w_gate, routing, w2=self.w_up, out=hidden, in_map=1, out_map=0, gate=self.gate,
                      gate_limit=s.limit, exact=exact)
-        if s.top == 1:
-            ops.moe_gemm(hidden, self.w_down, routing, 1, out=residual, in_map=0, out_map=2, weight=1.0, exact=exact)
+        if routing.many:
+            y = torch.empty((A, residual.shape[1]), dtype=torch.float32, device=xb.device)
+            ops.moe_gemm(hidden, self.w_down, routing, out=y, in_map=0, out_map=0, exact=exact)
+            ops.moe_combine(y, residual, s.top, 1.0 / s.top, place_of=routing.place_of)
+        elif s.top == 1:
+            ops.moe_gemm(hidden, self.w_down, routing, out=residual, in_map=0, out_map=2, weight=1.0, exact=exact)
         else:
             y = torch.empty((A, residual.shape[1]), dtype=torch.float32, device=xb.device)
-            ops.moe_gemm(hidden, self.w_down, routing, s.top, out=y, in_map=0, out_map=1, exact=exact)
+            ops.moe_gemm(hidden, self.w_down, routing, out=y, in_map=0, out_map=1, exact=exact)
             ops.moe_combine(y, residual, s.top, 1.0 / s.top)
         return None
 

@@ -25,7 +25,7 @@ def built(miforax_folders):
 
     def get(name, dtype):
         if (name, dtype) not in cache:
-            model = load_model(miforax_folders[name], dtype, torch.device(DEV), max_positions=512)
+            model = load_model(miforax_folders[name], dtype, torch.device(DEV), max_positions=1024)
             cache[(name, dtype)] = (model, build_runner(model, page_size=mt.CONFIGS[name][2], pool_tokens=1024,
                                                         max_requests=4, graphs=False))
         return cache[(name, dtype)]
@@ -61,7 +61,7 @@ def test_feed_forwards_alone(name, dtype, built, miforax_folders):
     model, runner = built(name, dtype)
     act = torch.float32 if dtype == "float32" else torch.bfloat16
     torch.manual_seed(3)
-    for T in (1, 7, 45):
+    for T in (1, 7, 45, 600):  # 600 rows give MB's experts enough rows each for the tiles of many rows
         toks = mt.prompt(name, T, seed=T)
         ctx = runner.prepare([StepEntry("ff", toks, [])])
         xb = (torch.randn(T, cfg["width"]) * 1.5).to(act)  # large enough that the experts' clamps bite

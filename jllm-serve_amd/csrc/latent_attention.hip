@@ -57,13 +57,16 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   }
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int sub = lane & 15, q4 = lane >> 4;
-  const int v = wave * 16 + sub;
+  // A single row of at most 16 heads is 16 query vectors, one wave's worth: then all four waves take the same query
+  // vectors and every fourth group of 16 keys each, and merge at the end in the order of the waves.
+  const bool kpar = r_hi == r_lo && HB <= 16;
+  const int v = kpar ? sub : wave * 16 + sub;
   const int my_r = r_lo + v / HB, my_h = hb * HB + v % HB;
   const bool live = my_r <= r_hi && my_h < H;
   const int my_pos = p_lo + v / HB;
   const int my_first = window > 0 ? max(0, my_pos + 1 - window) : 0;
   // the keys this wave's rows can see (a wave without a live query vector only helps to load)
-  const int wr_lo = r_lo + (wave * 16) / HB, wr_hi = min(r_hi, r_lo + (wave * 16 + 15) / HB);
+  const int wr_lo = kpar ? r_lo : r_lo + (wave * 16) / HB, wr_hi = kpar ? r_lo : min(r_hi, r_lo + (wave * 16 + 15) / HB);
   const bool wave_live = wr_lo <= r_hi;
   const int w_lo = window > 0 ? max(0, p_lo + (wr_lo - r_lo) + 1 - window) : 0;
   const int w_hi = p_lo + (wr_hi - r_lo);  // (with a split the loop's own bounds narrow these further)
@@ -119,6 +122,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       for (int st = 0; st < LM_KEYS / 16; ++st) {
         const int k0 = c0 + st * 16;
         if (k0 + 15 < w_lo || k0 > w_hi) continue;  // none of these keys is seen by a row of this wave
+        if (kpar && st != wave) continue;            // another wave's keys
         floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f}, sc2 = floatx4{0.f, 0.f, 0.f, 0.f};  // two chains of dependent MFMAs
         const bf16_t* krow = Kb + (st * 16 + sub) * LD + 8 * q4;
 #pragma unroll
@@ -161,9 +165,40 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
     __syncthreads();  // the other buffer is whole, and everyone is done with this one
     cur ^= 1;
   }
-  if (!live) return;
   l1 += __shfl_xor(l1, 16, 64);
   l1 += __shfl_xor(l1, 32, 64);
+  if (kpar) {  // the loop's last barrier has passed: the key buffers now carry the merge
+    constexpr int MS = 2 + 4 * RT;
+    float* mrg = (float*)lm_smem;  // [LM_WAVES - 1][64][MS]
+    if (wave > 0) {
+      float* d = mrg + (size_t)((wave - 1) * 64 + lane) * MS;
+      d[0] = m1, d[1] = l1;
+#pragma unroll
+      for (int j = 0; j < RT; ++j)
+        if (j < r16) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) d[2 + 4 * j + i] = acc[j][i];
+        }
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll 1
+    for (int w = 0; w < LM_WAVES - 1; ++w) {
+      const float* src = mrg + (size_t)(w * 64 + lane) * MS;
+      const float om = src[0], ol = src[1];
+      const float mn = fmaxf(m1, om);
+      const float a = lm_exp_diff(m1, mn), b = lm_exp_diff(om, mn);
+      l1 = l1 * a + ol * b;
+#pragma unroll
+      for (int j = 0; j < RT; ++j)
+        if (j < r16) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[j][i] = acc[j][i] * a + src[2 + 4 * j + i] * b;
+        }
+      m1 = mn;
+    }
+  }
+  if (!live) return;
   if (split > 0) {
     float* dst = part + (((size_t)(row0 + my_r) * H + my_h) * gridDim.z + blockIdx.z) * (R + 4);  // R sums, maximum, sum
     if (q4 == 0) dst[R] = m1, dst[R + 1] = l1;
@@ -187,7 +222,9 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       *(u32x2*)(o + 16 * j) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
 }
 
-// merges the key ranges of one (row, head) in ascending order; one wave per (row, head)
+// merges the key ranges of one (row, head); one wave per (row, head). Lane z first takes range z's maximum and sum (all
+// ranges at once: n_z <= 64), the wave agrees on the overall maximum and every range's weight, and then the weighted
+// sums are added in ascending order of the ranges with several ranges' loads in flight.
 __global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part, const int* __restrict__ positions,
                                                                    int H, int R, int window, int split, int n_z,
                                                                    const float* __restrict__ sink, bf16_t* __restrict__ out,
@@ -196,32 +233,29 @@ __global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float*
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
   const int s0 = first / split;
-  float m = -INFINITY, l = 0.f;
+  const int n_valid = min(n_z, pos / split - s0 + 1);  // the ranges that hold keys of this row
+  const float* base = part + ((size_t)t * H + h) * n_z * (R + 4);
+  float pm = -INFINITY, pl = 0.f;
+  if (lane < n_valid) pm = base[(size_t)lane * (R + 4) + R], pl = base[(size_t)lane * (R + 4) + R + 1];
+  float m = wave_max(pm);
+  const float sk = sink ? sink[h] : -INFINITY;
+  m = fmaxf(m, sk);
+  const float wz = lm_exp_diff(pm, m);
+  float l = wave_sum(pl * wz) + (sink ? __expf(sk - m) : 0.f);
   float acc[8];  // R <= 512
 #pragma unroll
   for (int a = 0; a < 8; ++a) acc[a] = 0.f;
-  for (int z = 0; z < n_z; ++z) {
-    if ((s0 + z) * split > pos) break;
-    const float* src = part + (((size_t)t * H + h) * n_z + z) * (R + 4);
-    const float pm = src[R], pl = src[R + 1];
-    const float mn = fmaxf(m, pm);
-    const float ca = lm_exp_diff(m, mn), cb = lm_exp_diff(pm, mn);
-    l = l * ca + pl * cb;
+#pragma unroll 4
+  for (int z = 0; z < n_valid; ++z) {
+    const float w = __shfl(wz, z, 64);
+    const float* src = base + (size_t)z * (R + 4);
 #pragma unroll
     for (int a = 0; a < 8; ++a) {
       const int d = lane + 64 * a;
-      if (d < R) acc[a] = acc[a] * ca + src[d] * cb;
+      if (d < R) acc[a] = fmaf(src[d], w, acc[a]);
     }
-    m = mn;
   }
-  float ca = 1.0f;
-  if (sink) {
-    const float sk = sink[h];
-    const float mn = fmaxf(m, sk);
-    ca = lm_exp_diff(m, mn);
-    l = l * ca + __expf(sk - mn);
-  }
-  const float inv = ca / l;
+  const float inv = 1.0f / l;
 #pragma unroll
   for (int a = 0; a < 8; ++a) {
     const int d = lane + 64 * a;
@@ -271,7 +305,7 @@ extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, in
   const size_t smem = (size_t)2 * LM_KEYS * LD * sizeof(bf16_t);  // two buffers that take turns
   // `split` > 0: every tile is a single row (the caller's promise), whose keys are cut into absolute ranges of `split`
   // keys over n_z workgroups; `part` holds rows x H x n_z x (R + 4) floats
-  if (split > 0 && ((split & 63) || n_z < 1 || n_z > 65535 || !part)) JLLM_FAIL("latent_attention: ranges of %d keys over %d workgroups", split, n_z);
+  if (split > 0 && ((split & 63) || n_z < 1 || n_z > 64 || !part)) JLLM_FAIL("latent_attention: ranges of %d keys over %d workgroups", split, n_z);
   dim3 grid(n_tiles, n_hb * (split > 0 ? 1 : n_rg), split > 0 ? n_z : 1);
   int rc;
   if (R <= 64 && dkp <= 128)

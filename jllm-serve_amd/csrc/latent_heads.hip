@@ -55,7 +55,7 @@ __global__ __launch_bounds__(LHM_WAVES * 64) void latent_heads_mfma_kernel(
   for (int rb = 0; rb < RB; ++rb)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[rb][b] = floatx4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
+#pragma unroll 4
   for (int k0 = 0; k0 < K; k0 += 32) {
     const bool in_k = k0 + 8 * q4 < K;
     u32x4 xf[RB], wf[4];

@@ -982,6 +982,9 @@ def _latent_split(rows: int, heads: int, window: int, max_ctx: int):
         return 0, 1
     split = max(LATENT_SPLIT_MIN, -(-(-(-span // want)) // 64) * 64)
     n_z = -(-span // split) + 1  # a span of that many keys touches at most this many absolute ranges
+    while n_z > 64:  # the merge takes up to 64 ranges
+        split *= 2
+        n_z = -(-span // split) + 1
     return (split, n_z) if n_z > 2 else (0, 1)
 
 

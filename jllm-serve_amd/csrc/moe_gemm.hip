@@ -9,8 +9,8 @@
 
 #define MM_WAVES 4
 
-// RB: 16-row blocks of a tile (tiles of 16 rows for steps with few rows per expert, of 64 where experts get many: a
-// weight fragment then meets four activation fragments)
+// RB: 16-row blocks of a tile. Built with RB = 1: steps that give the experts many rows each go through the grouped form
+// of the tiled product (gemm_mfma.hip) instead, which shares its operands through LDS.
 template <bool GATED, int RB>
 __global__ __launch_bounds__(MM_WAVES * 64) void moe_gemm_mfma_kernel(
     const bf16_t* __restrict__ A, int lda, const bf16_t* __restrict__ W, const bf16_t* __restrict__ W2,
@@ -94,7 +94,7 @@ extern "C" int jllm_moe_gemm_bf16(const void* A, int a_dtype, int lda, const voi
   if (max_tiles <= 0) return 0;
   if (a_dtype != JLLM_BF16 || w_dtype != JLLM_BF16) return 1;
   if (N <= 0 || K <= 0 || lda < K || ldo < N) JLLM_FAIL("moe_gemm: N %d K %d lda %d ldo %d", N, K, lda, ldo);
-  if (tile_rows != 16 && tile_rows != 64) JLLM_FAIL("moe_gemm: this kernel takes tiles of 16 or 64 rows, the route made %d", tile_rows);
+  if (tile_rows != 16) JLLM_FAIL("moe_gemm: this kernel takes tiles of 16 rows, the route made %d", tile_rows);
   JLLM_TAKE_GATE("moe_gemm", epilogue, gate_limit, gs);
   if ((epilogue != 0 && epilogue != 2) || (epilogue == 2) != (W2 != nullptr)) JLLM_FAIL("moe_gemm: epilogue %d", epilogue);
   if (in_map < 0 || in_map > 1 || out_map < 0 || out_map > 2) JLLM_FAIL("moe_gemm: maps %d / %d", in_map, out_map);
@@ -109,12 +109,8 @@ extern "C" int jllm_moe_gemm_bf16(const void* A, int a_dtype, int lda, const voi
 #define MM_LAUNCH(GATED, RB)                                                                                                    \
   moe_gemm_mfma_kernel<GATED, RB><<<grid, MM_WAVES * 64, 0, stream>>>((const bf16_t*)A, lda, (const bf16_t*)W, (const bf16_t*)W2, out, \
                                                                       out_dtype, ldo, N, K, sorted, tiles, top, in_map, out_map, weight, gs)
-  if (W2 && tile_rows == 64)
-    MM_LAUNCH(true, 4);
-  else if (W2)
+  if (W2)
     MM_LAUNCH(true, 1);
-  else if (tile_rows == 64)
-    MM_LAUNCH(false, 4);
   else
     MM_LAUNCH(false, 1);
 #undef MM_LAUNCH

@@ -222,14 +222,15 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       *(u32x2*)(o + 16 * j) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
 }
 
-// merges the key ranges of one (row, head); one wave per (row, head). Lane z first takes range z's maximum and sum (all
-// ranges at once: n_z <= 64), the wave agrees on the overall maximum and every range's weight, and then the weighted
-// sums are added in ascending order of the ranges with several ranges' loads in flight.
-__global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float* __restrict__ part, const int* __restrict__ positions,
+// merges the key ranges of one (row, head); four waves per (row, head), a thread owns dims tid and tid + 256. Lane z of
+// every wave first takes range z's maximum and sum (all ranges at once: n_z <= 64), the wave agrees on the overall
+// maximum and every range's weight, and then the weighted sums are added in ascending order of the ranges with eight
+// ranges' loads in flight.
+__global__ __launch_bounds__(256) void latent_attention_merge_kernel(const float* __restrict__ part, const int* __restrict__ positions,
                                                                    int H, int R, int window, int split, int n_z,
                                                                    const float* __restrict__ sink, bf16_t* __restrict__ out,
                                                                    int ldo) {
-  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63;
   const int pos = positions[t];
   const int first = window > 0 ? max(0, pos + 1 - window) : 0;
   const int s0 = first / split;
@@ -242,23 +243,21 @@ __global__ __launch_bounds__(64) void latent_attention_merge_kernel(const float*
   m = fmaxf(m, sk);
   const float wz = lm_exp_diff(pm, m);
   float l = wave_sum(pl * wz) + (sink ? __expf(sk - m) : 0.f);
-  float acc[8];  // R <= 512
-#pragma unroll
-  for (int a = 0; a < 8; ++a) acc[a] = 0.f;
-#pragma unroll 4
+  float acc[2] = {0.f, 0.f};  // R <= 512
+#pragma unroll 8
   for (int z = 0; z < n_valid; ++z) {
     const float w = __shfl(wz, z, 64);
     const float* src = base + (size_t)z * (R + 4);
 #pragma unroll
-    for (int a = 0; a < 8; ++a) {
-      const int d = lane + 64 * a;
+    for (int a = 0; a < 2; ++a) {
+      const int d = threadIdx.x + 256 * a;
       if (d < R) acc[a] = fmaf(src[d], w, acc[a]);
     }
   }
   const float inv = 1.0f / l;
 #pragma unroll
-  for (int a = 0; a < 8; ++a) {
-    const int d = lane + 64 * a;
+  for (int a = 0; a < 2; ++a) {
+    const int d = threadIdx.x + 256 * a;
     if (d < R) stf(out + (size_t)t * ldo + (size_t)h * R, d, acc[a] * inv);
   }
 }
@@ -317,7 +316,7 @@ extern "C" int jllm_latent_attention_bf16(const void* qa, int ldq, void* out, in
   if (rc != 0) return rc;
   JLLM_CHECK_LAUNCH("latent_attention");
   if (split > 0) {
-    latent_attention_merge_kernel<<<dim3(n_tiles, H), 64, 0, stream>>>(part, positions, H, R, window, split, n_z, sink, (bf16_t*)out, ldo);
+    latent_attention_merge_kernel<<<dim3(n_tiles, H), 256, 0, stream>>>(part, positions, H, R, window, split, n_z, sink, (bf16_t*)out, ldo);
     JLLM_CHECK_LAUNCH("latent_attention_merge");
   }
   return 0;

@@ -47,11 +47,9 @@ def inverse_frequencies(spec: RopeSpec) -> np.ndarray:
         low_dim, high_dim = correction_dim(s.beta_fast), correction_dim(s.beta_slow)
         low = max(math.floor(low_dim) if s.truncate else low_dim, 0)
         high = min(math.ceil(high_dim) if s.truncate else high_dim, dim - 1)
-        if low == high:
-            high += 0.001
         extra = f
         inter = 1.0 / (s.factor * np.power(float(spec.theta), (2.0 * i) / dim))
-        ramp = np.clip((i - low) / (high - low), 0.0, 1.0)
+        ramp = np.clip((i - low) / max(high - low, 0.001), 0.0, 1.0)  # a ramp of no width is a step
         return inter * ramp + extra * (1 - ramp)
     raise ValueError(f"unknown rope scaling '{s.kind}'")
 

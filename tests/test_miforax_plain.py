@@ -52,7 +52,8 @@ def test_parser_refuses(edit, text):
 
 @pytest.mark.parametrize("rot", [{"base": 1e4, "dims": 16}, {"base": 5e5, "dims": 32, "scaling": mt._yarn(4.0, 64)},
                                  {"base": 100.0, "dims": 8, "scaling": mt._yarn(0.5, 8, fast=4.0, slow=2.0)},
-                                 {"base": 1e6, "dims": 64, "scaling": mt._yarn(8.0, 4096, fast=32.0, slow=1.0)}])
+                                 {"base": 1e6, "dims": 64, "scaling": mt._yarn(8.0, 4096, fast=32.0, slow=1.0)},
+                                 {"base": 50.0, "dims": 16, "scaling": mt._yarn(3.0, 40, fast=1.0, slow=6.0)}])  # a ramp that ends before it starts
 def test_rotation_table_of_the_engine_is_the_plain_one(rot):
     from jllm_serve_amd.config.miforax import _rope
     from jllm_serve_amd.parts.rope import rope_table

@@ -1,8 +1,12 @@
 // Latent attention on the matrix cores, bf16: portions of prompts and single decoded rows through one kernel.
 //
 // All heads of a row attend over the same cached rows (Dk = R + Dr numbers per position, the first R of which are also
-// the values), so the query vectors of many heads and rows share every key they read. A workgroup of four waves takes
-// 64 query vectors of one run of rows of one request (HB heads x 64 / HB consecutive rows; a wave owns 16 of them),
+// the values), so the query vectors of many heads and rows share every key they read. A workgroup takes 64 query
+// vectors of one run of rows of one request (HB heads x 64 / HB consecutive rows). It has eight waves: waves w and w + 4
+// own the same 16 query vectors and both compute their scores and softmax, but each keeps only one half of the latent's
+// accumulators (a 512-wide latent is 128 registers per lane; one wave holding all of it and its queries left no
+// registers to have LDS reads in flight, and timestamps showed every fragment read's latency standing in front of its
+// product: 2,900 cycles for the 18 score products of 16 keys). The workgroup
 // walks the keys its rows can see in blocks of 64 aligned to absolute positions, and stages each block once in LDS as
 // it lies in the cache (two buffers take turns: the next block travels while this one is multiplied). Per 16 keys a wave computes
 //   S^T = K . Q^T   (MFMA 16x16x32; K fragments from LDS, Q^T in registers): a lane then holds four keys' scores of
@@ -23,7 +27,8 @@
 #include "common.h"
 #include "mfma.h"
 
-#define LM_WAVES 4
+#define LM_WAVES 8
+#define LM_QW 4  // waves with query vectors of their own; waves 4..7 repeat them for the other half of the latent
 #define LM_KEYS 64
 #define LM_TILE_ROWS 16
 
@@ -60,17 +65,20 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   // A single row of at most 16 heads is 16 query vectors, one wave's worth: then all four waves take the same query
   // vectors and every fourth group of 16 keys each, and merge at the end in the order of the waves.
   const bool kpar = r_hi == r_lo && HB <= 16;
-  const int v = kpar ? sub : wave * 16 + sub;
+  const int qwave = wave & (LM_QW - 1), rhalf = wave / LM_QW;
+  const int v = kpar ? sub : qwave * 16 + sub;
   const int my_r = r_lo + v / HB, my_h = hb * HB + v % HB;
   const bool live = my_r <= r_hi && my_h < H;
   const int my_pos = p_lo + v / HB;
   const int my_first = window > 0 ? max(0, my_pos + 1 - window) : 0;
   // the keys this wave's rows can see (a wave without a live query vector only helps to load)
-  const int wr_lo = kpar ? r_lo : r_lo + (wave * 16) / HB, wr_hi = kpar ? r_lo : min(r_hi, r_lo + (wave * 16 + 15) / HB);
+  const int wr_lo = kpar ? r_lo : r_lo + (qwave * 16) / HB, wr_hi = kpar ? r_lo : min(r_hi, r_lo + (qwave * 16 + 15) / HB);
   const bool wave_live = wr_lo <= r_hi;
   const int w_lo = window > 0 ? max(0, p_lo + (wr_lo - r_lo) + 1 - window) : 0;
   const int w_hi = p_lo + (wr_hi - r_lo);  // (with a split the loop's own bounds narrow these further)
   const int dks = (Dk + 31) >> 5, r16 = R >> 4;
+  constexpr int RTH = (RT + 1) / 2;  // accumulators of one wave: its half of the latent's 16-dim blocks
+  const int j_lo = rhalf ? (r16 + 1) / 2 : 0, nj = rhalf ? r16 - (r16 + 1) / 2 : (r16 + 1) / 2;
   const int psh = __builtin_ctz(page_size);
   const int* tbl = block_table + (size_t)req * max_blocks;
 
@@ -83,30 +91,30 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       qf[j] = (live && j < dks && d < Dk) ? *(const u32x4*)(qrow + d) : u32x4{0u, 0u, 0u, 0u};
     }
   }
-  floatx4 acc[RT];
+  floatx4 acc[RTH];
 #pragma unroll
-  for (int j = 0; j < RT; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < RTH; ++j) acc[j] = floatx4{0.f, 0.f, 0.f, 0.f};
   float m1 = -INFINITY, l1 = 0.f;
   // A block of 64 keys goes global -> registers -> LDS. All of a thread's pieces are requested together (first their
   // table entries, then the rows: two latencies a block, not two per piece), and the next block's are requested before
   // this block is multiplied, into the other of two LDS buffers: one barrier per block.
-  // four threads to a key row (256 threads, 64 rows): a thread's pieces are 16 bytes at (tid % 4) * 16 + 64 i of its row:
-  // one table entry and one address per block
-  constexpr int CPT = DKS;
-  static_assert(LM_WAVES * 64 == 4 * LM_KEYS, "four threads stage a key row");
+  // eight threads to a key row (512 threads, 64 rows): a thread's pieces are 16 bytes at (tid % 8) * 16 + 128 i of its
+  // row: one table entry and one address per block
+  constexpr int CPT = (DKS + 1) / 2;
+  static_assert(LM_WAVES * 64 == 8 * LM_KEYS, "eight threads stage a key row");
   uint4 staged[CPT];
-  const int srow = threadIdx.x >> 2, scol = (threadIdx.x & 3) * 8;
+  const int srow = threadIdx.x >> 3, scol = (threadIdx.x & 7) * 8;
   auto fetch = [&](int blk) {
     const int key = min(max(blk * LM_KEYS + srow, kb), ke);  // a key outside the range is masked below and reads one inside it
     const bf16_t* src = cache + ((((size_t)tbl[key >> psh]) << psh) + (key & (page_size - 1))) * Dk + scol;
 #pragma unroll
-    for (int i = 0; i < CPT; ++i) staged[i] = (i < dks && scol + 32 * i < Dk) ? *(const uint4*)(src + 32 * i) : uint4{0u, 0u, 0u, 0u};
+    for (int i = 0; i < CPT; ++i) staged[i] = (scol + 64 * i < Dk) ? *(const uint4*)(src + 64 * i) : uint4{0u, 0u, 0u, 0u};
   };
   auto put = [&](bf16_t* buf) {
     bf16_t* dst = buf + srow * LD + scol;
 #pragma unroll
     for (int i = 0; i < CPT; ++i)
-      if (i < dks) *(uint4*)(dst + 32 * i) = staged[i];
+      if (scol + 64 * i < dks * 32) *(uint4*)(dst + 64 * i) = staged[i];
   };
   const int blk_last = ke >> 6;
   int cur = 0;
@@ -122,7 +130,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
       for (int st = 0; st < LM_KEYS / 16; ++st) {
         const int k0 = c0 + st * 16;
         if (k0 + 15 < w_lo || k0 > w_hi) continue;  // none of these keys is seen by a row of this wave
-        if (kpar && st != wave) continue;            // another wave's keys
+        if (kpar && st != qwave) continue;           // another wave's keys
         floatx4 sc = floatx4{0.f, 0.f, 0.f, 0.f}, sc2 = floatx4{0.f, 0.f, 0.f, 0.f};  // two chains of dependent MFMAs
         const bf16_t* krow = Kb + (st * 16 + sub) * LD + 8 * q4;
 #pragma unroll
@@ -145,7 +153,7 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
           const float alpha = lm_exp_diff(m1, mx);
           l1 *= alpha;
 #pragma unroll
-          for (int j = 0; j < RT; ++j) acc[j] *= alpha;
+          for (int j = 0; j < RTH; ++j) acc[j] *= alpha;
           m1 = mx;
         }
         float p[4];
@@ -157,8 +165,8 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
         const u32x2 pb = u32x2{pack_bf16(p[0], p[1]), pack_bf16(p[2], p[3])};
         const bf16_t* v_tr = Kb + (st * 16 + 4 * q4 + (sub >> 2)) * LD + 4 * (sub & 3);
 #pragma unroll
-        for (int j = 0; j < RT; ++j)
-          if (j < r16) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * j), pb, acc[j]);
+        for (int j = 0; j < RTH; ++j)
+          if (j < nj) acc[j] = mfma16k16(lds_read_tr16(v_tr + 16 * (j_lo + j)), pb, acc[j]);
       }
     }
     if (blk < blk_last) put(Ks + (size_t)(cur ^ 1) * LM_KEYS * LD);
@@ -168,30 +176,30 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   l1 += __shfl_xor(l1, 16, 64);
   l1 += __shfl_xor(l1, 32, 64);
   if (kpar) {  // the loop's last barrier has passed: the key buffers now carry the merge
-    constexpr int MS = 2 + 4 * RT;
-    float* mrg = (float*)lm_smem;  // [LM_WAVES - 1][64][MS]
-    if (wave > 0) {
-      float* d = mrg + (size_t)((wave - 1) * 64 + lane) * MS;
+    constexpr int MS = 2 + 4 * RTH;
+    float* mrg = (float*)lm_smem + (size_t)rhalf * (LM_QW - 1) * 64 * MS;  // [2][LM_QW - 1][64][MS]
+    if (qwave > 0) {
+      float* d = mrg + (size_t)((qwave - 1) * 64 + lane) * MS;
       d[0] = m1, d[1] = l1;
 #pragma unroll
-      for (int j = 0; j < RT; ++j)
-        if (j < r16) {
+      for (int j = 0; j < RTH; ++j)
+        if (j < nj) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) d[2 + 4 * j + i] = acc[j][i];
         }
     }
     __syncthreads();
-    if (wave > 0) return;
+    if (qwave > 0) return;
 #pragma unroll 1
-    for (int w = 0; w < LM_WAVES - 1; ++w) {
+    for (int w = 0; w < LM_QW - 1; ++w) {
       const float* src = mrg + (size_t)(w * 64 + lane) * MS;
       const float om = src[0], ol = src[1];
       const float mn = fmaxf(m1, om);
       const float a = lm_exp_diff(m1, mn), b = lm_exp_diff(om, mn);
       l1 = l1 * a + ol * b;
 #pragma unroll
-      for (int j = 0; j < RT; ++j)
-        if (j < r16) {
+      for (int j = 0; j < RTH; ++j)
+        if (j < nj) {
 #pragma unroll
           for (int i = 0; i < 4; ++i) acc[j][i] = acc[j][i] * a + src[2 + 4 * j + i] * b;
         }
@@ -201,10 +209,10 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   if (!live) return;
   if (split > 0) {
     float* dst = part + (((size_t)(row0 + my_r) * H + my_h) * gridDim.z + blockIdx.z) * (R + 4);  // R sums, maximum, sum
-    if (q4 == 0) dst[R] = m1, dst[R + 1] = l1;
+    if (q4 == 0 && rhalf == 0) dst[R] = m1, dst[R + 1] = l1;
 #pragma unroll
-    for (int j = 0; j < RT; ++j)
-      if (j < r16) *(floatx4*)(dst + 16 * j + 4 * q4) = acc[j];
+    for (int j = 0; j < RTH; ++j)
+      if (j < nj) *(floatx4*)(dst + 16 * (j_lo + j) + 4 * q4) = acc[j];
     return;
   }
   float ca = 1.0f;
@@ -217,9 +225,9 @@ __global__ __launch_bounds__(LM_WAVES * 64) void latent_attention_mfma_kernel(
   const float inv = ca / l1;
   bf16_t* o = out + (size_t)(row0 + my_r) * ldo + (size_t)my_h * R + 4 * q4;
 #pragma unroll
-  for (int j = 0; j < RT; ++j)
-    if (j < r16)
-      *(u32x2*)(o + 16 * j) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
+  for (int j = 0; j < RTH; ++j)
+    if (j < nj)
+      *(u32x2*)(o + 16 * (j_lo + j)) = u32x2{pack_bf16(acc[j][0] * inv, acc[j][1] * inv), pack_bf16(acc[j][2] * inv, acc[j][3] * inv)};
 }
 
 // merges the key ranges of one (row, head); four waves per (row, head), a thread owns dims tid and tid + 256. Lane z of

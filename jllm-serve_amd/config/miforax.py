@@ -10,7 +10,8 @@ A Miforax config names its design with ``"architecture": "Miforax"`` and lists i
   key), ``rot`` (``base``, ``dims``, optional ``scaling`` with ``factor``, ``original``, ``fast``, ``slow``: YaRN) and
   optionally ``kv_from: j``: the layer reads layer j's cached latent and has no down-projection of its own;
 * a feed-forward: ``kind`` ``dense`` (``ff``; gelu-tanh gate) or ``moe`` (``router.experts`` / ``router.top``,
-  ``expert.ff`` / ``expert.limit``, optional ``shared.ff`` / ``shared.limit``; experts come from a table by token id).
+  ``expert.ff`` / ``expert.limit``, optional ``shared.ff`` / ``shared.limit``; experts come from a table by token id; the
+  slope 1.702 of the experts' sigmoid is the design's and lives in the kernels' gate function).
 
 YaRN here: the frequencies blend between f_i and f_i / factor over the dimensions between the ``fast`` and ``slow``
 rotation counts of the ``original`` length, and cos and sin are multiplied by 0.1 ln(factor) + 1 whatever the factor;
@@ -24,9 +25,6 @@ from typing import Any, List, Mapping, Optional
 from .registry import register_architecture
 from .schema import (ConfigError, GatedMlpNames, GatedMlpSpec, LatentAttentionSpec, LayerSpec, ModelConfig, ModelNames,
                      NormSpec, RopeScaling, RopeSpec, ScheduleEntry, TableMoeSpec)
-
-SWISH_ALPHA = 1.702  # the design's sigmoid slope in its experts' gate; fixed, not a config key
-
 
 def _need(m: Any, key: str, where: str):
     if not isinstance(m, Mapping) or key not in m or m[key] is None:

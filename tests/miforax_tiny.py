@@ -3,7 +3,9 @@
 MF_A varies everything a layer can vary: a layer that borrows an earlier layer's cache and looks further back than
 that layer does, a layer without a window, a rotated key part only half of which is rotated, a layer without a
 feed-forward, experts with top = 2 and a shared expert, experts with top = 1 and none, rotation with and without YaRN.
-MF_B has sizes the matrix-core kernels take (multiples of 16 / 32 / 128), so its bfloat16 run goes through them.
+MF_B has sizes the matrix-core kernels take (multiples of 16 / 32 / 128), so its bfloat16 run goes through them. MF_C
+has odd sizes everywhere (one head, a value size of 5, an embedding scale of 1, a layer that borrows a cache and has no
+window, so that its owner, which has one, must keep every page).
 """
 import json
 import os
@@ -58,8 +60,18 @@ MF_B = {
     ],
 }
 
+# sizes that are multiples of nothing: every product and attention falls to the general kernels in bfloat16 too
+MF_C = {
+    "architecture": "Miforax", "vocab": 97, "width": 70, "norm": {"eps": 1e-6}, "embedding": {"scale": 1.0},
+    "layers": [
+        _layer(_mixer(3, 10, 6, 7, 18, 20, window=9, rot_dims=4, scaling=_yarn(1.5, 8, fast=8.0, slow=2.0)), _moe(4, 3, 12, 1.0, shared=(22, 2.0))),
+        _layer(_mixer(1, 12, 2, 5, 9, 11, base=77.0), {"kind": "dense", "ff": 50}),
+        _layer(_mixer(5, 6, 6, 9, 18, 20, rot_dims=4, scaling=_yarn(1.5, 8, fast=8.0, slow=2.0), kv_from=0), _moe(2, 2, 30, 0.5)),
+    ],
+}
+
 # name -> (config, weight seed, page size)
-CONFIGS = {"MA": (MF_A, 11, 8), "MB": (MF_B, 12, 16)}
+CONFIGS = {"MA": (MF_A, 11, 8), "MB": (MF_B, 12, 16), "MC": (MF_C, 13, 4)}
 
 
 def write_model(folder, cfg, seed, std=0.09, sink_std=1.5):

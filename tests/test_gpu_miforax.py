@@ -53,7 +53,7 @@ def close(got, want, dtype, what=""):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["MA", "MB"])
+@pytest.mark.parametrize("name", ["MA", "MB", "MC"])
 def test_feed_forwards_alone(name, dtype, built, miforax_folders):
     from jllm_serve_amd.engine.step import StepEntry
     cfg = mt.CONFIGS[name][0]
@@ -82,7 +82,7 @@ def test_feed_forwards_alone(name, dtype, built, miforax_folders):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["MA", "MB"])
+@pytest.mark.parametrize("name", ["MA", "MB", "MC"])
 def test_mixers_alone_through_the_cache(name, dtype, built, miforax_folders):
     """Every layer's mixer on random inputs: a portion from position 0, a second portion and single rows from the
     cache; a layer that borrows a cache reads what its owner stored from the owner's own input."""
@@ -249,7 +249,7 @@ def _replay(model, trace, page, shuffle=None):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["MA", "MB"])
+@pytest.mark.parametrize("name", ["MA", "MB", "MC"])
 def test_replays_match_plain_and_each_other(name, dtype, miforax_folders, plain_logits):
     """Whole prompts, the last tokens one by one (captured steps in bfloat16), portions down to two tokens, and mixed
     batches of up to four requests on a pool exactly as large as the busiest step with free pages in random order."""

@@ -195,7 +195,7 @@ extern "C" int jllm_latent_heads_generic(const void* in, int dtype, int ld_in, i
 // One workgroup of four waves per (row, GC heads). The row at position p sees keys [first, p], first = max(0, p + 1 -
 // window) with a window, else 0. Within a 64-key block a lane owns one key for the scores (ascending dims) and
 // 64-strided value dims for the weighted sum (ascending keys). All heads read the same rows.
-#define LA_MAX_ACC 8  // R <= 512
+#define LA_MAX_ACC 16  // R <= 1024
 #define LA_WAVES 4
 
 template <typename T>

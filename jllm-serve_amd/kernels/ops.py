@@ -819,7 +819,7 @@ def decode_attention_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
 
 # ------------------------------------------------------------------------------------------------ latent attention
 
-MAX_LATENT = 512       # the latent a cached row may hold (csrc/latent_generic.hip); the rotated key part comes on top
+MAX_LATENT = 1024      # the latent a cached row may hold (csrc/latent_generic.hip; the matrix-core kernel takes up to 512)
 
 
 def check_latent_shape(heads: int, kv_rank: int, rot_dim: int, rot_dims: int) -> None:

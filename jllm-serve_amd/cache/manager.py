@@ -84,7 +84,7 @@ class CacheEntryPlan:
 
     kv: Optional[PageSpec] = None  # None: this run owns no pages
     cache_from: Optional[int] = None  # reads the pages of that earlier run
-    state: Optional[StateSpec] = None
+    state: Optional[object] = None  # a StateSpec, or a tuple of them (the run then gets a tuple of tensors)
 
 
 @dataclass
@@ -95,7 +95,7 @@ class LayerSlot:
     rows: Dict[str, torch.Tensor] = field(default_factory=dict)  # row name -> [pages, *page shape] of this run
     page_size: int = 0
     writes: bool = True
-    state: Optional[torch.Tensor] = None  # [slots, *shape]
+    state: Optional[object] = None  # [slots, *shape], or a tuple of such tensors where the run declared several
 
 
 class KvGroup:
@@ -164,9 +164,15 @@ class CacheManager:
             if p.state is not None and allocate:
                 # one row beyond the request slots: the state of the padding rows of a captured step, which no live
                 # request ever holds (a mixer may read and write it like any other row)
-                slot.state = torch.zeros((max_requests + 1,) + tuple(p.state.shape), dtype=p.state.dtype, device=self.device)
-            self._state_tensors.append(slot.state)
+                many = isinstance(p.state, (tuple, list))
+                made = [torch.zeros((max_requests + 1,) + tuple(st.shape), dtype=st.dtype, device=self.device)
+                        for st in (p.state if many else (p.state,))]
+                slot.state = tuple(made) if many else made[0]
+                self._state_tensors += made
+            elif p.state is not None:
+                self._state_tensors.append(None)
             self.slots.append(slot)
+        self._has_state = any(p.state is not None for p in plans)
         self._free_state = list(range(max_requests - 1, -1, -1))
         self.padding_state_slot = max_requests
         for g in self.groups:
@@ -349,7 +355,7 @@ class CacheManager:
         rc = self.requests[rid]
         if length > rc.length or length < 0:
             raise ValueError(f"cannot truncate {rc.length} positions to {length}")
-        if length < rc.length and any(t is not None for t in self._state_tensors):
+        if length < rc.length and self._has_state:
             raise ValueError("a model with per-request state cannot be rewound")
         keep = -(-length // self.page_size)
         for gi, g in enumerate(self.groups):

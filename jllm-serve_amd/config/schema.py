@@ -41,7 +41,8 @@ class RopeScaling:
 
 @dataclass(frozen=True)
 class RopeSpec:
-    """One rotary table (model/RopeTable.java:20-52). ``pairing`` "half" rotates (i, i + rotary_dim/2)."""
+    """One rotary table (model/RopeTable.java:20-52). ``pairing`` "half" rotates (i, i + rotary_dim/2), "interleaved"
+    rotates (2i, 2i + 1); the table is the same for both, the mixer's kernels apply it."""
 
     rotary_dim: int
     theta: float
@@ -64,6 +65,16 @@ class NormSpec:
 
     eps: float
     kind: str = "rmsnorm"
+
+
+@dataclass(frozen=True)
+class LayerNormSpec:
+    """Layer norm with a weight and a bias: (x - mean) / sqrt(mean of squared deviations + eps) * w + b. The bias is the
+    tensor whose name is the weight's with ``bias_suffix`` added."""
+
+    eps: float
+    bias_suffix: str = ".b"
+    kind: str = "layernorm"
 
 
 # --------------------------------------------------------------------------- mixers
@@ -169,6 +180,104 @@ class LatentAttentionSpec:
     kind: str = "latent_attention"
 
 
+@dataclass(frozen=True)
+class WideAttentionNames:
+    """Tensor names of an attention whose keys and values have sizes of their own, under the mixer's prefix; a bias is
+    the weight's name with ``bias_suffix``, the gains of a norm over a whole projection the projection's name with
+    ``norm_suffix``."""
+
+    q: str = "q"
+    k: str = "k"
+    v: str = "v"
+    gate: str = "g"
+    o: str = "o"
+    bias_suffix: str = ".b"
+    norm_suffix: str = ".norm"
+    lambda_q: Tuple[str, ...] = ("lq1", "lq2")  # differential attention: the vectors whose products give lambda
+    lambda_k: Tuple[str, ...] = ("lk1", "lk2")
+
+
+@dataclass(frozen=True)
+class WideAttentionSpec:
+    """Causal grouped-query attention with a key size ``dim`` and a value size ``vdim`` of their own.
+
+    ``maps`` 1: ordinary. ``maps`` 2 (differential attention): every query head and every key head holds two maps laid
+    out [map 1 | map 2]; both are softmaxed alone over the same values and combined as a1 - lambda a2 with lambda =
+    exp(lq1 . lk1) - exp(lq2 . lk2) + ``diff``; each head's result is divided by its root mean square (``eps``) and
+    multiplied by 1 - ``diff``. ``qk_norm`` "whole": RMS norm with gains over the whole q projection and the whole k
+    projection before the heads are split. ``position``: index of a rotary table (applied with its pairing on the
+    first rotary_dim entries of every head) or None. ``softcap`` > 0: scores become softcap * tanh(score / softcap).
+    ``q_temp_every`` > 0: q at position p is multiplied by 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1).
+    ``out_gate``: the concatenated heads are multiplied by sigmoid(W_g h) before the output product."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    scale: float
+    eps: float
+    maps: int = 1
+    diff: float = 0.0
+    qk_norm: Optional[str] = None
+    position: Optional[int] = None
+    softcap: float = 0.0
+    q_temp_coef: float = 0.0
+    q_temp_every: int = 0
+    bias: bool = True
+    out_gate: bool = True
+    window: int = 0
+    names: WideAttentionNames = WideAttentionNames()
+    kind: str = "wide_attention"
+
+
+@dataclass(frozen=True)
+class GatedDeltaNames:
+    """Tensor names of a gated-delta-rule mixer under its prefix; a projection's convolution taps are its name with
+    ``conv_suffix``."""
+
+    q: str = "q"
+    k: str = "k"
+    v: str = "v"
+    beta: str = "b"
+    decay: str = "a"
+    a_log: str = "A_log"
+    dt_bias: str = "dt_bias"
+    norm: str = "norm"
+    gate: str = "g"
+    o: str = "o"
+    conv_suffix: str = ".conv"
+
+
+@dataclass(frozen=True)
+class GatedDeltaSpec:
+    """A recurrent mixer: per head a matrix S [dim, vdim] that decays, is corrected towards the new value along the new
+    key (the delta rule) and is read with the query. q and k have ``kv_heads`` heads of ``dim`` (value head h uses head
+    h / (heads / kv_heads)), v has ``heads`` heads of ``vdim``; q, k and v pass a causal convolution of ``conv`` taps per
+    channel and silu; q and k are made unit vectors (q also times dim^-1/2); the write strength is sigmoid(W_b h), the
+    decay exp(-exp(A_log) softplus(W_a h + dt_bias)) per head; each head's read-out is divided by its root mean square
+    (``eps``), multiplied by a gain shared by the heads and by silu(W_g h), and goes through W_o."""
+
+    heads: int
+    kv_heads: int
+    dim: int
+    vdim: int
+    conv: int
+    eps: float
+    names: GatedDeltaNames = GatedDeltaNames()
+    kind: str = "gated_delta"
+
+
+@dataclass(frozen=True)
+class ParallelMixerSpec:
+    """Mixers side by side on the same input: the result is the sum of ``scales[i]`` times branch i's output. Branch
+    i's tensors lie under the mixer's prefix + ``prefixes[i]``. At most one branch may own pages."""
+
+    branches: Tuple[Any, ...]
+    scales: Tuple[float, ...]
+    prefixes: Tuple[str, ...]
+    kind: str = "parallel"
+
+
 # --------------------------------------------------------------------------- feed-forwards
 
 
@@ -248,15 +357,32 @@ class LayerSpec:
     norm_in_name: str = "input_layernorm"  # under the prefix, without the ending
     norm_post_name: str = "post_attention_layernorm"
     name_ending: str = ".weight"
+    # arrangement "sandwich": x += norm_mixer_out(mixer(norm_in(x))); x += norm_ffn_out(ffn(norm_post(x)))
+    norm_mixer_out_name: str = ""
+    norm_ffn_out_name: str = ""
+    mixer_prefix: str = ""  # under the layer's prefix, for mixers whose tensor names are relative to it
+
+
+@dataclass(frozen=True)
+class StreamVector:
+    """A learned vector that is added to every row of the residual stream: row ``row`` of the tensor ``name``
+    [``rows``, hidden]."""
+
+    name: str
+    rows: int
+    row: int
 
 
 @dataclass(frozen=True)
 class ScheduleEntry:
     """One step of the layer schedule: run ``layer``; ``cache_from`` names an earlier schedule entry
-    whose cache this run reads instead of writing one of its own (None = its own cache)."""
+    whose cache this run reads instead of writing one of its own (None = its own cache); ``add_before``: a vector
+    that joins the stream right before this run (a layer that runs several times with one set of weights has a cache
+    or state per run, and may be told which pass it is in this way)."""
 
     layer: int
     cache_from: Optional[int] = None
+    add_before: Optional[StreamVector] = None
 
 
 @dataclass(frozen=True)

@@ -1,0 +1,132 @@
+// Layer norm with weight and bias over fp32 rows of the residual stream, alone or as the seam between two sublayers.
+//
+//   y = (x - mean(x)) / sqrt(mean((x - mean(x))^2) + eps) * w + b          all sums and the result in fp32
+//
+// One workgroup per row, the row in registers, two block sums in a fixed order (mean, then the squared deviations), so
+// a row's result depends on nothing but the row. One kernel does up to three things to a row, in this order:
+//   1. with `a`: the row t = s1 * a (+ s2 * a2) is normed with (w_post, b_post) and added into the residual row
+//      (a sublayer whose output passes a norm of its own before it joins the stream; two branches with fixed weights)
+//   2. with `add_vec`: a vector is added to the residual row (a learned offset for every row of the step)
+//   3. with `out`: the (new) residual row is normed with (w_next, b_next) into `out` for the next sublayer's products
+// With a row list, only 3 runs and row i of `out` is the norm of residual row rows[i] (the rows whose logits are wanted).
+#include <math.h>
+
+#include "common.h"
+
+#define LN_THREADS 256
+
+template <int VPT>
+__device__ __forceinline__ void ln_stats(const float (&v)[VPT], int d, float* red, float& mean, float& rstd, float eps) {
+  float s = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * LN_THREADS;
+    if (i < d) s += v[k];
+  }
+  mean = block_sum<LN_THREADS / 64>(s, red) / (float)d;
+  float q = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * LN_THREADS;
+    if (i < d) {
+      const float c = v[k] - mean;
+      q = fmaf(c, c, q);
+    }
+  }
+  const float var = block_sum<LN_THREADS / 64>(q, red) / (float)d;
+  rstd = (float)(1.0 / sqrt((double)(var + eps)));
+}
+
+template <typename TA, typename TW, typename TO, int VPT>
+__global__ __launch_bounds__(LN_THREADS) void layernorm_seam_kernel(
+    float* __restrict__ residual, const int* __restrict__ rows, int d, const TA* __restrict__ a, int lda,
+    const TA* __restrict__ a2, int lda2, float s1, float s2, const TW* __restrict__ w_post, const TW* __restrict__ b_post,
+    const TW* __restrict__ add_vec, const TW* __restrict__ w_next, const TW* __restrict__ b_next, float eps,
+    TO* __restrict__ out, int ldo) {
+  __shared__ float red[LN_THREADS / 64];
+  const int r = blockIdx.x;
+  const size_t src = rows ? (size_t)rows[r] : (size_t)r;
+  float* xr = residual + src * d;
+  float x[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int i = threadIdx.x + k * LN_THREADS;
+    x[k] = i < d ? xr[i] : 0.f;
+  }
+  if (a) {
+    float t[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int i = threadIdx.x + k * LN_THREADS;
+      t[k] = 0.f;
+      if (i < d) {
+        t[k] = s1 * ldf(a + (size_t)r * lda, i);
+        if (a2) t[k] = fmaf(s2, ldf(a2 + (size_t)r * lda2, i), t[k]);
+      }
+    }
+    float mean, rstd;
+    ln_stats<VPT>(t, d, red, mean, rstd, eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int i = threadIdx.x + k * LN_THREADS;
+      if (i < d) x[k] += (t[k] - mean) * rstd * ldf(w_post, i) + ldf(b_post, i);
+    }
+  }
+  if (add_vec) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int i = threadIdx.x + k * LN_THREADS;
+      if (i < d) x[k] += ldf(add_vec, i);
+    }
+  }
+  if (a || add_vec) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int i = threadIdx.x + k * LN_THREADS;
+      if (i < d) xr[i] = x[k];
+    }
+  }
+  if (out) {
+    float mean, rstd;
+    ln_stats<VPT>(x, d, red, mean, rstd, eps);
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int i = threadIdx.x + k * LN_THREADS;
+      if (i < d) stf(out + (size_t)r * ldo, i, (x[k] - mean) * rstd * ldf(w_next, i) + ldf(b_next, i));
+    }
+  }
+}
+
+// residual fp32 [*, d] contiguous; a, a2: [n, >= d] in a_dtype or null; weights, biases and the vector in w_dtype;
+// out [n, ldo] in out_dtype or null
+extern "C" int jllm_layernorm_seam(float* residual, const int* rows, int n, int d, const void* a, int lda, const void* a2,
+                                   int lda2, int a_dtype, float s1, float s2, const void* w_post, const void* b_post,
+                                   const void* add_vec, const void* w_next, const void* b_next, int w_dtype, float eps,
+                                   void* out, int out_dtype, int ldo, hipStream_t stream) {
+  if (n <= 0) return 0;
+  if (d <= 0 || d > LN_THREADS * 32) JLLM_FAIL("layernorm: rows of %d entries (this kernel takes 1..%d)", d, LN_THREADS * 32);
+  if (a && (!w_post || !b_post || lda < d || (a2 && lda2 < d))) JLLM_FAIL("layernorm: a branch without its norm or with short rows");
+  if (a2 && !a) JLLM_FAIL("layernorm: a second branch without a first");
+  if (out && (!w_next || !b_next || ldo < d)) JLLM_FAIL("layernorm: an output without its norm or with short rows");
+  if (rows && (a || add_vec)) JLLM_FAIL("layernorm: a row list goes with the output norm alone");
+  if (!a && !add_vec && !out) return 0;
+#define LN_LAUNCH(VPT)                                                                                                \
+  layernorm_seam_kernel<TA, TW, TO, VPT><<<n, LN_THREADS, 0, stream>>>(                                               \
+      residual, rows, d, (const TA*)a, lda, (const TA*)a2, lda2, s1, s2, (const TW*)w_post, (const TW*)b_post,        \
+      (const TW*)add_vec, (const TW*)w_next, (const TW*)b_next, eps, (TO*)out, ldo)
+  JLLM_DISPATCH_1(a_dtype, TA, {
+    JLLM_DISPATCH_1(w_dtype, TW, {
+      JLLM_DISPATCH_1(out_dtype, TO, {
+        if (d <= LN_THREADS * 4)
+          LN_LAUNCH(4);
+        else if (d <= LN_THREADS * 16)
+          LN_LAUNCH(16);
+        else
+          LN_LAUNCH(32);
+      })
+    })
+  })
+#undef LN_LAUNCH
+  JLLM_CHECK_LAUNCH("layernorm_seam");
+  return 0;
+}

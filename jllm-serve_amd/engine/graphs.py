@@ -110,7 +110,12 @@ class DecodeGraphs:
         sizes["max_context"] = ck  # launch shapes of the bucket, whatever the live requests hold
         ctx = r._context(dev, sizes, segments)
         ctx.segments = []  # a captured step must not depend on host-side facts of one batch
-        # once eagerly, so that nothing is loaded or configured for the first time inside the capture
+        # once eagerly, so that nothing is loaded or configured for the first time inside the capture. That run must
+        # leave no trace, since the replay that follows computes the same step again: keys and values land where the
+        # replay writes them anyway, but a state that is carried from token to token would move on twice, so every
+        # request of the eager run works on the state row of the padding requests (the upload in front of the first
+        # replay restores the real rows)
+        ctx.state_slots.fill_(r.cache.padding_state_slot)
         r.model.forward(ctx, r.cache.slots)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()

@@ -75,6 +75,12 @@ def _declare(lib) -> None:
         "jllm_moe_gemm_generic": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
         "jllm_moe_combine": [_P, _P, _I, _I, _I, _F, _P, _P],
         "jllm_copy_page_rows": [_P, _I, _I, _I, _I, _L, _I, _I, _I, _P],
+        "jllm_layernorm_seam": [_P, _P, _I, _I, _P, _I, _P, _I, _I, _F, _F, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _P],
+        "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
+        "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _P, _I, _I, _P],
+        "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
+        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -989,6 +995,269 @@ def _latent_split(rows: int, heads: int, window: int, max_ctx: int):
 
 
 # ------------------------------------------------------------------------------------------------ table-routed experts
+
+# ------------------------------------------------------------------------------------------------ layer norm
+
+
+def _same_type(what: str, *tensors):
+    have = [t for t in tensors if t is not None]
+    if any(t.dtype != have[0].dtype or not t.is_contiguous() for t in have):
+        raise KernelError(f"{what} must be contiguous tensors of one type")
+    return _code(have[0].dtype) if have else F32
+
+
+def layernorm_seam(residual: torch.Tensor, eps: float, *, a: Optional[torch.Tensor] = None,
+                   a2: Optional[torch.Tensor] = None, s1: float = 1.0, s2: float = 1.0, post=None,
+                   add_vec: Optional[torch.Tensor] = None, nxt=None, out_dtype: Optional[torch.dtype] = None,
+                   rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """What happens to the fp32 residual rows between two sublayers, in one launch, each part optional and in this
+    order: ``residual += layer_norm(s1 * a (+ s2 * a2); post)``; ``residual += add_vec``; and the layer norm of the
+    (new) rows with ``nxt`` as a new tensor of ``out_dtype``, which is returned. ``post`` and ``nxt`` are (weight,
+    bias) pairs. With ``rows`` (int32) only the last part runs, over the listed rows."""
+    _dev(residual, a, a2, add_vec, rows)
+    if residual.dtype != torch.float32 or residual.dim() != 2 or not residual.is_contiguous():
+        raise KernelError("the residual must be a contiguous fp32 [rows, width] tensor")
+    n, d = residual.shape
+    if rows is not None:
+        if a is not None or add_vec is not None:
+            raise KernelError("layernorm: a row list goes with the output norm alone")
+        n = rows.numel()
+        _i32(rows, n, "row list")
+    for t in (a, a2):
+        if t is not None:
+            _rows2d(t, "a sublayer's output")
+            if t.shape != (n, d):
+                raise KernelError(f"layernorm: a sublayer's output is {tuple(t.shape)}, the residual {(n, d)}")
+    if a is None and a2 is not None:
+        raise KernelError("layernorm: a second branch without a first")
+    if a is not None and a2 is not None and a2.dtype != a.dtype:
+        raise KernelError("layernorm: both branches must share a type")
+    if (a is not None) != (post is not None):
+        raise KernelError("layernorm: a sublayer's output and its norm come together")
+    vecs = [v for pair in (post, nxt) if pair is not None for v in pair] + ([add_vec] if add_vec is not None else [])
+    for v in vecs:
+        _dev(v)
+        if v.numel() != d:
+            raise KernelError(f"layernorm: a weight, bias or vector has {v.numel()} entries, the rows have {d}")
+    wd = _same_type("layernorm weights, biases and vectors", *vecs)
+    out = None
+    if nxt is not None:
+        out = activation_rows(n, d, out_dtype or torch.float32, residual.device)
+    if n == 0:
+        return out
+    _call("jllm_layernorm_seam", _ptr(residual), _ptr(rows), n, d, _ptr(a), a.stride(0) if a is not None else 0, _ptr(a2),
+          a2.stride(0) if a2 is not None else 0, _code(a.dtype) if a is not None else F32, float(s1), float(s2),
+          _ptr(post[0]) if post else None, _ptr(post[1]) if post else None, _ptr(add_vec),
+          _ptr(nxt[0]) if nxt else None, _ptr(nxt[1]) if nxt else None, wd, float(eps), _ptr(out),
+          _code(out.dtype) if out is not None else F32, out.stride(0) if out is not None else 0, _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ attention with sizes of its own
+
+
+MAX_VALUE_DIM = 512    # what the attention kernels for separate key and value sizes take (csrc/attention_dv.hip)
+
+
+def check_attention_dv_shape(heads: int, kv_heads: int, maps: int, dk: int, dv: int, rot_dims: int) -> None:
+    """Raises when the attention kernels for separate key and value sizes do not take these sizes (asked when a model
+    is built)."""
+    if heads <= 0 or kv_heads <= 0 or heads % kv_heads != 0 or maps not in (1, 2):
+        raise KernelError(f"attention: {heads} query heads over {kv_heads} kv heads with {maps} score maps")
+    if not 0 < dv <= MAX_VALUE_DIM or dk <= 0:
+        raise KernelError(f"attention: key size {dk}, value size {dv} (values of 1..{MAX_VALUE_DIM} are taken)")
+    if (heads + kv_heads) * maps * dk * 4 > 64 * 1024:
+        raise KernelError(f"attention: q and k of a row ({(heads + kv_heads) * maps * dk} entries) are more than the preparing kernel holds")
+    if rot_dims and (rot_dims < 2 or rot_dims > dk or rot_dims % 2):
+        raise KernelError(f"attention: a rotary width of {rot_dims} for heads of {dk} (even, 2..{dk}, is taken)")
+
+
+def _check_kv_pages(k_cache, v_cache, k_slots, v_heads, dk, dv, dtype):
+    if k_cache.dtype != dtype or not k_cache.is_contiguous() or k_cache.dim() != 4 or k_cache.shape[1] != k_slots or k_cache.shape[3] != dk:
+        raise KernelError(f"the key pages must be a contiguous [pages, {k_slots}, page_size, {dk}] tensor of the activations' type")
+    if v_cache.dtype != dtype or not v_cache.is_contiguous() or v_cache.dim() != 4 or v_cache.shape[1] != v_heads or v_cache.shape[3] != dv \
+            or v_cache.shape[2] != k_cache.shape[2] or v_cache.shape[0] != k_cache.shape[0]:
+        raise KernelError(f"the value pages must be a contiguous [pages, {v_heads}, page_size, {dv}] tensor beside the key pages")
+
+
+def qkv_prepare(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torch.Tensor], heads: int, kv_heads: int,
+                maps: int, dk: int, dv: int, k_cache: torch.Tensor, v_cache: torch.Tensor, *,
+                gq: Optional[torch.Tensor] = None, gk: Optional[torch.Tensor] = None, eps: float = 0.0,
+                cos: Optional[torch.Tensor] = None, sin: Optional[torch.Tensor] = None, rot_dims: int = 0,
+                temp_coef: float = 0.0, temp_every: int = 0) -> None:
+    """In place on the first columns of ``qkv`` rows [q: heads x maps x dk | k: kv_heads x maps x dk | v: kv_heads x
+    dv]: with ``gq``/``gk`` an RMS norm with those gains over the whole of q and the whole of k; with ``rot_dims`` the
+    rotation of the pairs (2i, 2i + 1) among the first ``rot_dims`` entries of every q and k head by the table rows of
+    the positions; with ``temp_every`` q times 1 + temp_coef * ln(floor((p + 1) / temp_every) + 1); then k and v go to
+    the rows' ``slots`` in the pages (``slots`` None or negative entries: nothing is stored)."""
+    _dev(qkv, positions, slots, gq, gk, cos, sin, k_cache, v_cache)
+    _rows2d(qkv, "qkv")
+    T = qkv.shape[0]
+    q_slots, k_slots = heads * maps, kv_heads * maps
+    if qkv.shape[1] < (q_slots + k_slots) * dk + kv_heads * dv:
+        raise KernelError(f"qkv rows have {qkv.shape[1]} entries, fewer than q, k and v take")
+    _i32(positions, T, "positions")
+    _i32(slots, T, "slots")
+    _tables(cos, sin, rot_dims)
+    if (gq is None) != (gk is None):
+        raise KernelError("the norm over the projections takes gains for both q and k")
+    if gq is not None and (gq.numel() != q_slots * dk or gk.numel() != k_slots * dk):
+        raise KernelError(f"the gains of the norm over the projections must have {q_slots * dk} and {k_slots * dk} entries")
+    gd = _same_type("the gains of q and k", gq, gk)
+    _check_kv_pages(k_cache, v_cache, k_slots, kv_heads, dk, dv, qkv.dtype)
+    _call("jllm_qkv_prepare", _ptr(qkv), qkv.stride(0), _code(qkv.dtype), T, _ptr(positions), _ptr(slots), q_slots, k_slots,
+          kv_heads, dk, dv, _ptr(gq), _ptr(gk), gd, float(eps), _ptr(cos), _ptr(sin), int(rot_dims), float(temp_coef),
+          int(temp_every), _ptr(k_cache), _ptr(v_cache), k_cache.shape[2], _stream())
+
+
+def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
+                 row_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, maps: int, dk: int, dv: int,
+                 scale: float, *, softcap: float = 0.0, window: int = 0, out_dtype: Optional[torch.dtype] = None,
+                 meta=None, exact: bool = False) -> torch.Tensor:
+    """Causal attention of every row of ``q`` [T, heads x maps x dk] over its request's pages, keys [pages, kv_heads x
+    maps, page_size, dk] and values [pages, kv_heads, page_size, dv]: map m of head h reads key slot (h / (heads /
+    kv_heads)) * maps + m and value head h / (heads / kv_heads). Scores (q . k) * scale, capped as softcap * tanh(score
+    / softcap) when ``softcap`` > 0. Returns [T, heads x maps x dv] in ``out_dtype`` (default: q's)."""
+    _dev(q, k_cache, v_cache, block_table, row_req, positions)
+    _rows2d(q, "q")
+    T = q.shape[0]
+    if q.shape[1] != heads * maps * dk:
+        raise KernelError(f"q rows have {q.shape[1]} entries, expected {heads * maps * dk}")
+    _check_kv_pages(k_cache, v_cache, kv_heads * maps, kv_heads, dk, dv, q.dtype)
+    if block_table.dtype != torch.int32 or block_table.dim() != 2 or not block_table.is_contiguous():
+        raise KernelError("block table must be a contiguous int32 [requests, max_blocks] tensor")
+    _i32(row_req, T, "row -> request map")
+    _i32(positions, T, "positions")
+    out = torch.empty((T, heads * maps * dv), dtype=out_dtype or q.dtype, device=q.device)
+    if T == 0:
+        return out
+    if not exact and _fast_attention_dv is not None and _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions,
+                                                                        heads, kv_heads, maps, dk, dv, scale, softcap, window, meta):
+        return out
+    if not exact:
+        _count("general", "jllm_attention_dv_generic")
+    _call("jllm_attention_dv_generic", _ptr(q), q.stride(0), _code(q.dtype), _ptr(out), out.stride(0), _code(out.dtype),
+          _ptr(k_cache), _ptr(v_cache), _ptr(block_table), block_table.shape[1], _ptr(row_req), _ptr(positions), T, heads,
+          kv_heads, maps, dk, dv, k_cache.shape[2], int(window), float(scale), float(softcap), _stream())
+    return out
+
+
+_fast_attention_dv = None
+
+
+def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: torch.dtype, *, lam: float = 0.0,
+                 normed: bool = False, eps: float = 0.0, norm_mul: float = 1.0, gain: Optional[torch.Tensor] = None,
+                 gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """From the attention's rows [T, heads x maps x dv] to the output product's input [T, heads x dv]: with two maps
+    o = a1 - lam * a2; ``normed``: o / sqrt(mean(o^2) + eps) * norm_mul per head (times ``gain`` [dv]); with ``gate``
+    ([T, heads x dv], a view with any row stride) times sigmoid(gate)."""
+    _dev(att, gain, gate)
+    _rows2d(att, "attention rows")
+    T = att.shape[0]
+    if att.shape[1] != heads * maps * dv:
+        raise KernelError(f"attention rows have {att.shape[1]} entries, expected {heads * maps * dv}")
+    if gate is not None:
+        _rows2d(gate, "gate")
+        if gate.shape != (T, heads * dv):
+            raise KernelError(f"the gate is {tuple(gate.shape)}, expected {(T, heads * dv)}")
+    if gain is not None and (gain.numel() != dv or not gain.is_contiguous()):
+        raise KernelError(f"the heads' gain must have {dv} entries")
+    out = activation_rows(T, heads * dv, out_dtype, att.device)
+    if T == 0:
+        return out
+    _call("jllm_heads_finish", _ptr(att), att.stride(0), _code(att.dtype), T, heads, maps, dv, float(lam), 1 if normed else 0,
+          float(eps), float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
+          gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, _ptr(out),
+          out.stride(0), _code(out.dtype), _stream())
+    return out
+
+
+# ------------------------------------------------------------------------------------------------ gated delta rule
+
+
+MAX_CONV_TAPS = 16
+
+
+def check_gated_delta_shape(heads: int, kv_heads: int, dk: int, dv: int, taps: int) -> None:
+    """Raises when the delta-rule kernels do not take these sizes (asked when a model is built): a head's state of
+    dk x dv fp32 numbers lives in the registers of one workgroup."""
+    if heads <= 0 or kv_heads <= 0 or heads % kv_heads != 0:
+        raise KernelError(f"gated delta rule: {heads} heads over {kv_heads} key heads")
+    if not 1 <= taps <= MAX_CONV_TAPS:
+        raise KernelError(f"gated delta rule: a convolution of {taps} taps (1..{MAX_CONV_TAPS} are taken)")
+    if dk <= 0 or not 0 < dv <= 1024:
+        raise KernelError(f"gated delta rule: key size {dk}, value size {dv}")
+    parts = 1
+    while parts * 2 * dv <= 256 and parts * 2 <= dk and parts < 32:
+        parts *= 2
+    while -(-dk // parts) > 64 and parts * 2 * dv <= 1024 and parts < 32:
+        parts *= 2
+    if -(-dk // parts) > 64 or 2 * (2 * dk + 2 * parts * dv + dv) * 4 > 64 * 1024:
+        raise KernelError(f"gated delta rule: a state of {dk} x {dv} per head does not fit a workgroup")
+
+
+def short_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor,
+               n_requests: int) -> torch.Tensor:
+    """silu of a causal convolution over time per channel on the first C columns of ``x`` [T, >= C] (a view with any
+    row stride), ``taps`` [C, K] with the last column for the current row. A request's rows are consecutive and in
+    order; the inputs in front of its first row of this step come from ``state`` [slots, K - 1, C] (fp32, oldest
+    first) at the request's slot, and the state then moves on by the step's rows. Returns [T, C]."""
+    _dev(x, taps, state, row_req, state_slots)
+    _rows2d(x, "convolution input")
+    T = x.shape[0]
+    if taps.dim() != 2 or not taps.is_contiguous():
+        raise KernelError("convolution taps must be a contiguous [channels, taps] tensor")
+    C, K = taps.shape
+    if x.shape[1] < C:
+        raise KernelError(f"convolution input rows have {x.shape[1]} entries for {C} channels")
+    if state.dtype != torch.float32 or not state.is_contiguous() or (K > 1 and (state.dim() != 3 or state.shape[1:] != (K - 1, C))):
+        raise KernelError(f"the convolution's state must be a contiguous fp32 [slots, {K - 1}, {C}] tensor")
+    _i32(row_req, T, "row -> request map")
+    _i32(state_slots, n_requests, "state slots")
+    y = torch.empty((T, C), dtype=x.dtype, device=x.device)
+    if T == 0:
+        return y
+    _call("jllm_short_conv", _ptr(x), x.stride(0), _ptr(y), y.stride(0), _code(x.dtype), T, int(n_requests), C, K, _ptr(taps),
+          _code(taps.dtype), _ptr(state), _ptr(row_req), _ptr(state_slots), _stream())
+    return y
+
+
+def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, gate_off: int, a_off: int, b_off: int, a_log: torch.Tensor,
+                dt_bias: torch.Tensor, gain: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor,
+                state_slots: torch.Tensor, n_requests: int, heads: int, kv_heads: int, dk: int, dv: int,
+                eps: float) -> torch.Tensor:
+    """The gated delta rule over the step's rows, request by request and token by token, from and into ``state``
+    [slots, heads, dk, dv] (fp32). ``qkv`` [T, kv_heads x dk | kv_heads x dk | heads x dv] are the convolved q, k, v;
+    ``proj`` rows hold, at the given offsets, the output gate (heads x dv) and the inputs a and b of decay and write
+    strength (heads each). Per head: q and k become unit vectors (q also / sqrt(dk)); beta = sigmoid(b); g = exp(-exp(
+    a_log) softplus(a + dt_bias)); S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q; the result is o / sqrt(
+    mean(o^2) + eps) * gain * silu(gate), [T, heads x dv]."""
+    _dev(qkv, proj, a_log, dt_bias, gain, state, row_req, state_slots)
+    _rows2d(qkv, "convolved q, k, v")
+    _rows2d(proj, "projection rows")
+    T = qkv.shape[0]
+    if proj.shape[0] != T or proj.dtype != qkv.dtype:
+        raise KernelError("the projection rows and the convolved rows must agree in rows and type")
+    if qkv.shape[1] != 2 * kv_heads * dk + heads * dv:
+        raise KernelError(f"convolved rows have {qkv.shape[1]} entries, expected {2 * kv_heads * dk + heads * dv}")
+    if max(gate_off + heads * dv, a_off + heads, b_off + heads) > proj.shape[1] or min(gate_off, a_off, b_off) < 0:
+        raise KernelError("gate, a or b lie outside the projection rows")
+    if a_log.numel() != heads or dt_bias.numel() != heads or gain.numel() != dv:
+        raise KernelError(f"a_log and dt_bias must have {heads} entries, the gain {dv}")
+    wd = _same_type("a_log, dt_bias and the gain", a_log, dt_bias, gain)
+    if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dk, dv):
+        raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dk}, {dv}] tensor")
+    _i32(row_req, T, "row -> request map")
+    _i32(state_slots, n_requests, "state slots")
+    out = activation_rows(T, heads * dv, qkv.dtype, qkv.device)
+    if T == 0:
+        return out
+    _call("jllm_gated_delta", _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(gate_off), int(a_off), int(b_off),
+          _code(qkv.dtype), _ptr(a_log), _ptr(dt_bias), _ptr(gain), wd, _ptr(state), _ptr(out), out.stride(0), _ptr(row_req),
+          _ptr(state_slots), T, int(n_requests), heads, kv_heads, dk, dv, float(eps), _stream())
+    return out
+
+
 
 MOE_TILE_ROWS = 16      # rows of one expert that a workgroup of the grouped products takes in steps of few rows ...
 MOE_TILE_ROWS_MANY = 128  # ... and where the experts get many rows each (portions of prompts): the tiled product's tile

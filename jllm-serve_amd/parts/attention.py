@@ -75,6 +75,8 @@ class GqaAttention(Part):
         self.prefix = prefix
         self.build = build
         self.position = positions[spec.position] if spec.position is not None else None
+        if getattr(self.position, "pairing", "half") != "half":
+            raise ValueError(f"{prefix}: this mixer's kernels rotate the pairs (i, i + rotary_dim / 2) only")
         rot = self.position.rotary() if self.position is not None else None
         try:  # sizes that no kernel takes are refused here, when the model is built, not at the first step
             ops.check_attention_shape(spec.heads, spec.kv_heads, spec.head_dim, rot[2] if rot is not None else 0)

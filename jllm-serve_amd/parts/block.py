@@ -12,6 +12,8 @@ parts; a part that knows nothing of this works as before):
 """
 from __future__ import annotations
 
+import torch
+
 from .base import Part, part_factory, register_part
 
 
@@ -19,7 +21,8 @@ class PreNormBlock(Part):
     def __init__(self, spec, prefix, build, positions):
         ending = getattr(spec, "name_ending", ".weight")
         self.norm_in = part_factory("norm", spec.norm.kind)(spec.norm, build.hidden, f"{prefix}.{spec.norm_in_name}{ending}", build)
-        self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, prefix, build, positions)
+        mixer_prefix = f"{prefix}.{spec.mixer_prefix}" if getattr(spec, "mixer_prefix", "") else prefix
+        self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, mixer_prefix, build, positions)
         if spec.ffn is None:  # a layer of a mixer alone: no second norm, no feed-forward
             self.norm_post = self.ffn = None
             self.parts = (self.norm_in, self.mixer)
@@ -51,7 +54,7 @@ class PreNormBlock(Part):
     @staticmethod
     def _input(norm, consumer, x, promise):
         if getattr(consumer, "takes_normed_rows", False) and hasattr(norm, "defer"):
-            if promise is not None and promise.x is x and promise.gain is getattr(norm, "gain", None):
+            if promise is not None and getattr(promise, "x", None) is x and promise.gain is getattr(norm, "gain", None):
                 return promise
             return norm.defer(x)
         return norm.forward(x)
@@ -78,3 +81,97 @@ class PreNormBlock(Part):
 
 
 register_part("arrangement", "prenorm", PreNormBlock, replace=True)
+
+
+def sublayer_output(part, xb, step, slot, width):
+    """A mixer's or feed-forward's output as fp32 rows of its own, [rows, width]: its ``output`` method where it has
+    one, else what it adds into a cleared tensor."""
+    args = (step,) if slot is None else (step, slot)
+    if hasattr(part, "output"):
+        return part.output(xb, *args)
+    out = torch.empty((step.n_tokens, width), dtype=torch.float32, device=xb.device).zero_()
+    part.forward(xb, out, *args)
+    return out
+
+
+class SandwichBlock(Part):
+    """A norm in front of and behind each sublayer: x += norm_mixer_out(mixer(norm_in(x))); x += norm_ffn_out(ffn(
+    norm_post(x))). Where the norm part offers a ``seam`` (parts/norm.py: LayerNorm), the norm of a sublayer's output,
+    its add into the stream, a vector that joins the stream before the next layer, and the next sublayer's input norm
+    are one launch, handed on as the next block's input."""
+
+    chains_norms = True
+    takes_stream_vector = True  # forward(..., add_after=) adds that vector to the stream as its last act
+
+    def __init__(self, spec, prefix, build, positions):
+        ending = getattr(spec, "name_ending", ".weight")
+        make = part_factory("norm", spec.norm.kind)
+
+        def norm(name):
+            if not name:
+                raise ValueError(f"{prefix}: the sandwich arrangement names four norms")
+            return make(spec.norm, build.hidden, f"{prefix}.{name}{ending}", build)
+
+        self.width = build.hidden
+        self.norm_in = norm(spec.norm_in_name)
+        self.norm_mixer_out = norm(spec.norm_mixer_out_name)
+        mixer_prefix = f"{prefix}.{spec.mixer_prefix}" if getattr(spec, "mixer_prefix", "") else prefix
+        self.mixer = part_factory("mixer", spec.mixer.kind)(spec.mixer, mixer_prefix, build, positions)
+        if spec.ffn is None:
+            self.norm_post = self.norm_ffn_out = self.ffn = None
+            self.parts = (self.norm_in, self.mixer, self.norm_mixer_out)
+        else:
+            self.norm_post = norm(spec.norm_post_name)
+            self.norm_ffn_out = norm(spec.norm_ffn_out_name)
+            self.ffn = part_factory("ffn", spec.ffn.kind)(spec.ffn, prefix, build)
+            self.parts = (self.norm_in, self.mixer, self.norm_mixer_out, self.norm_post, self.ffn, self.norm_ffn_out)
+        self.capturable = all(getattr(p, "capturable", True) for p in self.parts)
+
+    def weight_specs(self):
+        return [w for p in self.parts for w in p.weight_specs()]
+
+    def load(self, get):
+        for p in self.parts:
+            p.load(get)
+
+    def cache_spec(self):
+        return self.mixer.cache_spec()
+
+    def state_spec(self):
+        return self.mixer.state_spec()
+
+    def step_planners(self):
+        return [pl for p in self.parts for pl in (p.step_planners() if hasattr(p, "step_planners") else [])]
+
+    @staticmethod
+    def _join(norm, x, branch, add_vec, then):
+        """x += norm(branch) (+ add_vec); returns then's norm of the new x, or None when nobody prepared it."""
+        if hasattr(norm, "seam") and (then is None or hasattr(then, "seam")):
+            return norm.seam(x, [branch], [1.0], add_vec=add_vec, then=then)
+        x += norm.forward(branch).float()
+        if add_vec is not None:
+            x += add_vec.float()
+        return None
+
+    def forward(self, x, step, slot, normed_in=None, next_norm=None, add_after=None):
+        """``normed_in``: norm_in of x as the block before left it (a tensor) or None; ``next_norm``: the norm part that
+        reads x next; ``add_after``: a vector that joins the stream behind this layer. Returns ``next_norm`` of the new
+        x when the last seam prepared it."""
+        xb = normed_in if isinstance(normed_in, torch.Tensor) else self.norm_in.forward(x)
+        then, vec = (next_norm, add_after) if self.ffn is None else (self.norm_post, None)
+        scales = getattr(getattr(self.mixer, "spec", None), "scales", ())
+        if hasattr(self.mixer, "outputs") and len(scales) == 2 and hasattr(self.norm_mixer_out, "seam") \
+                and (then is None or hasattr(then, "seam")):
+            # two weighted branches: their sum is taken inside the seam's launch
+            xb = self.norm_mixer_out.seam(x, self.mixer.outputs(xb, step, slot), list(scales), add_vec=vec, then=then)
+        else:
+            xb = self._join(self.norm_mixer_out, x, sublayer_output(self.mixer, xb, step, slot, self.width), vec, then)
+        if self.ffn is None:
+            return xb
+        if xb is None:
+            xb = self.norm_post.forward(x)
+        branch = sublayer_output(self.ffn, xb, step, None, self.width)
+        return self._join(self.norm_ffn_out, x, branch, add_after, next_norm)
+
+
+register_part("arrangement", "sandwich", SandwichBlock, replace=True)

@@ -53,5 +53,12 @@ class GatedMlp(Part):
         ops.gemm(h, self.w_down, out=residual, epilogue=ops.EPI_ADD, exact=self.build.exact)
         return None
 
+    def output(self, xb, step):
+        """The feed-forward's output as fp32 rows of its own, for an arrangement that norms it before the add."""
+        import torch
+        h = ops.gemm(xb, self.w_gate, w2=self.w_up, epilogue=ops.EPI_GATED, out_dtype=self.build.dtype,
+                     exact=self.build.exact, gate=self.gate, gate_limit=self.limit)
+        return ops.gemm(h, self.w_down, out_dtype=torch.float32, exact=self.build.exact)
+
 
 register_part("ffn", "gated_mlp", GatedMlp, replace=True)

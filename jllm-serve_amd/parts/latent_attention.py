@@ -59,6 +59,8 @@ class LatentAttention(Part):
         self.prefix = prefix
         self.build = build
         self.position = positions[spec.position] if spec.position is not None else None
+        if getattr(self.position, "pairing", "half") != "half":
+            raise ValueError(f"{prefix}: this mixer's kernels rotate the pairs (i, i + rotary_dim / 2) only")
         rot = self.position.rotary() if self.position is not None else None
         self.rot_dims = rot[2] if rot is not None else 0
         try:

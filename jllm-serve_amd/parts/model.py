@@ -38,6 +38,13 @@ class DecoderModel:
                                                                       config.names.final_norm, self.build)
         self.embed = None
         self.lm_head = None
+        # vectors that join the stream before a run (config: ScheduleEntry.add_before), by tensor name
+        self.stream_vector_rows = {}
+        for e in config.schedule:
+            if e.add_before is not None:
+                self.stream_vector_rows[e.add_before.name] = e.add_before.rows
+        self.stream_vectors = {}
+        self.watch = None  # a function (run, x) called with the stream after every run (tests, debugging)
         # a part that walks the step's requests on the host sets ``capturable = False``; then decode steps are
         # never recorded as graphs
         self.capturable = all(getattr(l, "capturable", True) for l in self.layers)
@@ -49,6 +56,7 @@ class DecoderModel:
         specs = [WeightSpec(c.names.embed, (c.vocab, c.hidden))]
         for p in self.positions:  # a position encoding may have tensors of its own (a learned table)
             specs += p.weight_specs() if hasattr(p, "weight_specs") else []
+        specs += [WeightSpec(name, (rows, c.hidden), init="bias") for name, rows in self.stream_vector_rows.items()]
         for l in self.layers:
             specs += l.weight_specs()
         specs += self.final_norm.weight_specs()
@@ -66,6 +74,7 @@ class DecoderModel:
         for p in self.positions:
             if hasattr(p, "load"):
                 p.load(get)
+        self.stream_vectors = {name: get(name) for name in self.stream_vector_rows}
         for l in self.layers:
             l.load(get)
         self.final_norm.load(get)
@@ -85,6 +94,9 @@ class DecoderModel:
         """What the layers want to know about every batch (engine/step.py runs each distinct planner once per step)."""
         return [pl for l in self.layers for pl in (l.step_planners() if hasattr(l, "step_planners") else [])]
 
+    def _stream_vector(self, v):
+        return self.stream_vectors[v.name][v.row]
+
     # -------------------------------------------------------------------------------------------- forward
 
     def forward(self, step, slots) -> torch.Tensor:
@@ -95,15 +107,31 @@ class DecoderModel:
                 p.embed_add(x, step)
         schedule = self.config.schedule
         carry = None  # the next block's input norm, when the block before prepared it (parts/block.py)
+        added = False  # this run's vector already joined the stream (the block before added it on its way out)
         for run, e in enumerate(schedule):
             layer = self.layers[e.layer]
+            if e.add_before is not None and not added:
+                ops.layernorm_seam(x, 0.0, add_vec=self._stream_vector(e.add_before))
+                carry = None
+            added = False
             if not getattr(layer, "chains_norms", False):
                 layer.forward(x, step, slots[run])
                 carry = None
-                continue
-            nxt = self.layers[schedule[run + 1].layer] if run + 1 < len(schedule) else None
-            next_norm = getattr(nxt, "norm_in", None) if getattr(nxt, "chains_norms", False) else None
-            carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm)
+            else:
+                nxt_e = schedule[run + 1] if run + 1 < len(schedule) else None
+                nxt = self.layers[nxt_e.layer] if nxt_e is not None else None
+                next_norm = getattr(nxt, "norm_in", None) if getattr(nxt, "chains_norms", False) else None
+                if nxt_e is not None and nxt_e.add_before is not None and self.watch is None \
+                        and getattr(layer, "takes_stream_vector", False):
+                    carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm,
+                                          add_after=self._stream_vector(nxt_e.add_before))
+                    added = True
+                else:
+                    if nxt_e is not None and nxt_e.add_before is not None:
+                        next_norm = None  # the stream changes before the next block reads it
+                    carry = layer.forward(x, step, slots[run], normed_in=carry, next_norm=next_norm)
+            if self.watch is not None:
+                self.watch(run, x)
         if step.n_selected == 0:
             return torch.empty((0, self.config.vocab), dtype=torch.float32, device=self.device)
         xs = self.final_norm.forward(x, rows=step.selected)

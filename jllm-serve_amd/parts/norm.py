@@ -1,7 +1,8 @@
-"""RMSNorm: y = (x * rsqrt(mean(x^2) + eps)) * g over fp32 rows (cpu/VectorKernels.java:630-634)."""
+"""RMSNorm: y = (x * rsqrt(mean(x^2) + eps)) * g over fp32 rows (cpu/VectorKernels.java:630-634), and layer norm with a
+weight and a bias: y = (x - mean) / sqrt(mean((x - mean)^2) + eps) * w + b."""
 from __future__ import annotations
 
-from ..config.schema import NormSpec
+from ..config.schema import LayerNormSpec, NormSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import BuildContext, Part, register_part
@@ -35,3 +36,55 @@ class RMSNorm(Part):
 
 
 register_part("norm", "rmsnorm", RMSNorm, replace=True)
+
+
+class LayerNorm(Part):
+    """Mean and variance in fp32 over fp32 rows. Beside ``forward`` it offers the seam between two sublayers as one
+    launch (``seam``): the norm of a sublayer's output added into the stream, a vector added to the stream, and the
+    next sublayer's input norm, each optional."""
+
+    def __init__(self, spec: LayerNormSpec, dim: int, weight_name: str, build: BuildContext):
+        self.eps = float(spec.eps)
+        self.dim = dim
+        self.weight_name = weight_name
+        self.bias_name = weight_name + spec.bias_suffix
+        self.out_dtype = build.dtype
+        self.gain = self.bias = None
+
+    def weight_specs(self):
+        return [WeightSpec(self.weight_name, (self.dim,), init="gain"), WeightSpec(self.bias_name, (self.dim,), init="bias")]
+
+    def load(self, get):
+        self.gain, self.bias = get(self.weight_name), get(self.bias_name)
+        if self.gain.dtype != self.bias.dtype:
+            self.gain, self.bias = self.gain.float(), self.bias.float()
+
+    def forward(self, x, rows=None):
+        return ops.layernorm_seam(x, self.eps, nxt=(self.gain, self.bias), out_dtype=self.out_dtype, rows=rows)
+
+    def seam(self, residual, branches, scales, add_vec=None, then=None):
+        """``residual += this norm of (sum_i scales[i] * branches[i])`` (one or two branches, [rows, width] each);
+        then ``residual += add_vec``; returns ``then``'s norm of the new rows (``then``: a LayerNorm part or None)."""
+        if not 1 <= len(branches) <= 2 or len(scales) != len(branches):
+            raise ValueError("the seam takes one or two branches with a scale each")
+        a2 = branches[1] if len(branches) == 2 else None
+        s2 = scales[1] if len(branches) == 2 else 0.0
+        vecs = [self.gain, self.bias]
+        nxt = None
+        if then is not None:
+            if then.eps != self.eps:
+                raise ValueError("the norms of one seam share their eps")
+            nxt = (then.gain, then.bias)
+            vecs += list(nxt)
+        if add_vec is not None:
+            vecs.append(add_vec)
+        if any(v.dtype != self.gain.dtype for v in vecs):  # one launch takes one type for all of them
+            out = ops.layernorm_seam(residual, self.eps, a=branches[0], a2=a2, s1=scales[0], s2=s2, post=(self.gain, self.bias))
+            if add_vec is not None:
+                ops.layernorm_seam(residual, self.eps, add_vec=add_vec)
+            return then.forward(residual) if then is not None else None
+        return ops.layernorm_seam(residual, self.eps, a=branches[0], a2=a2, s1=scales[0], s2=s2, post=(self.gain, self.bias),
+                                  add_vec=add_vec, nxt=nxt, out_dtype=then.out_dtype if then is not None else None)
+
+
+register_part("norm", "layernorm", LayerNorm, replace=True)

@@ -3,7 +3,8 @@
 model/Rope.java:24-38: inverse frequencies in double, ``cos[p, i] = (float)(cos(p * inv[i]) * amp)``;
 :122-167 the frequencies (plain ``theta^(-2i/rotary_dim)``, ``linear`` divides by the factor, ``llama3``
 blends by wavelength); :190-208 YaRN's ramp between extrapolation and interpolation; :75-85 the amplitude.
-The mixers rotate the pair (i, i + rotary_dim/2) by entry i ("half" pairing, model/RopeTable.java:9-18).
+The mixers rotate the pair (i, i + rotary_dim/2) by entry i ("half" pairing, model/RopeTable.java:9-18) or the pair
+(2i, 2i + 1) ("interleaved"); the table is the same, ``pairing`` tells the mixer which of its kernels' forms to use.
 """
 from __future__ import annotations
 
@@ -75,9 +76,10 @@ def rope_table(spec: RopeSpec, positions: int):
 
 class RotaryPosition(Part):
     def __init__(self, spec: RopeSpec, build: BuildContext):
-        if spec.pairing != "half":
-            raise ValueError(f"rotary pairing '{spec.pairing}' is not built (only 'half')")
+        if spec.pairing not in ("half", "interleaved"):
+            raise ValueError(f"rotary pairing '{spec.pairing}' is not built ('half' and 'interleaved' are)")
         self.spec = spec
+        self.pairing = spec.pairing
         cos, sin = rope_table(spec, build.max_positions)
         self.cos = torch.from_numpy(cos).to(build.device)
         self.sin = torch.from_numpy(sin).to(build.device)

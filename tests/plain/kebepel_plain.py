@@ -155,8 +155,8 @@ def short_convolution(x: torch.Tensor, taps: torch.Tensor) -> torch.Tensor:
     T, C = x.shape
     K = taps.shape[1]
     y = torch.zeros_like(x)
-    for j in range(K):
-        y[j:] += x[:T - j] * taps[:, K - 1 - j] if j else x * taps[:, K - 1]
+    for j in range(min(K, T)):
+        y[j:] += x[:T - j] * taps[:, K - 1 - j]
     return y
 
 

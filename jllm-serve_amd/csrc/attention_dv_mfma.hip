@@ -1,0 +1,302 @@
+// The attention of attention_dv.hip on the matrix cores, bf16 cache, for portions of prompts and single rows alike
+// (flash style: no score matrix in memory, running maximum and sum in fp32, the output in fp32).
+//
+// Grid (query slot, tile). A tile is up to 128 consecutive rows of one request (4 waves x 32 rows); the caller lists the
+// tiles as (request, first row, rows, position of the first row; a negative position means "the row's own entry of
+// the positions array", for steps whose shape is fixed before their positions are known), the ones with the most keys
+// first. Keys are walked in blocks of 64 aligned to absolute positions. Per block the workgroup stages the key slot's
+// K [64][dk] and the value head's V [64][dv] in LDS as they lie in the cache (two buffers: the next block's loads
+// are in flight while this one is multiplied); places outside the tile's visible range are stored as zeros and
+// their table entries are never read.
+//
+// Each wave computes the transposed scores S^T[key][row] = K Q^T (v_mfma_f32_32x32x16_bf16, A = K from LDS, B = Q
+// in registers), so a lane owns one query row: maximum and sum are in-lane reductions plus one exchange between the
+// half-waves. A cap on the scores (cap * tanh(s * scale / cap)) is applied to the accumulators before the softmax.
+// The probabilities, rounded to bf16, are already laid out as the B operand of O^T[dim][row] += V^T P^T, whose A
+// operand is read from V with the transposing LDS load (ds_read_b64_tr_b16). dk and dv are independent: dk in steps
+// of 16 (the K loop), dv in blocks of 32 (the accumulators), both up to 256.
+#include <math.h>
+
+#include "common.h"
+#include "mfma.h"
+
+#define AT_KEYS 64
+
+template <int DK16, int DB>
+__global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention_dv_tiles_kernel(
+    const bf16_t* __restrict__ q, int ldq, float* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
+    const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
+    const int* __restrict__ positions, int maps, int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window,
+    float scale, float softcap) {
+  constexpr int DK = DK16 * 16;
+  constexpr int DVP = DB * 32;
+  constexpr int KLD = DK + 8;
+  constexpr int VLD = DVP + 32;
+  constexpr int KSZ = AT_KEYS * KLD;
+  constexpr int VSZ = AT_KEYS * VLD;
+  constexpr int KCH = (AT_KEYS * DK16 * 2 + 255) / 256;  // 16-byte pieces of K per thread and block
+  constexpr int VPC = DVP / 8;                            // 16-byte pieces of a V row (the padded width)
+  constexpr int VCH = (AT_KEYS * VPC + 255) / 256;
+  extern __shared__ __align__(16) unsigned char smem_raw[];
+  bf16_t* Ks = (bf16_t*)smem_raw;  // [2][KSZ]
+  bf16_t* Vs = Ks + 2 * KSZ;       // [2][VSZ]
+  const int* tile = tiles + (size_t)blockIdx.y * 4;
+  const int req = tile[0], row0 = tile[1], nrows = tile[2];
+  const int pos0 = tile[3] >= 0 ? tile[3] : positions[row0];
+  const int s = blockIdx.x;
+  const int vh = s / per_kv;
+  const int ks_ = vh * maps + s % maps;
+  const int tid = threadIdx.x;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+  const int qi = lane & 31, half = lane >> 5;
+  const int wq = wave * 32 + qi;
+  const int pos_q = pos0 + min(wq, nrows - 1);
+  const int first_q = window > 0 ? max(0, pos_q + 1 - window) : 0;
+  const int* tbl = block_table + (size_t)req * max_blocks;
+  const int k_lo = window > 0 ? max(0, pos0 + 1 - window) : 0;
+  const int k_hi = pos0 + nrows - 1;
+  const int wave_lo_pos = pos0 + min(nrows - 1, wave * 32);
+  const int wave_hi = pos0 + min(nrows - 1, wave * 32 + 31);
+  const int wave_first = window > 0 ? max(0, wave_hi + 1 - window) : 0;
+  const bool wave_on = wave * 32 < nrows;
+  u32x4 qf[DK16];
+  {
+    const bf16_t* qr = q + (size_t)(row0 + min(wq, nrows - 1)) * ldq + (size_t)s * DK + half * 8;
+#pragma unroll
+    for (int i = 0; i < DK16; ++i) qf[i] = *(const u32x4*)(qr + i * 16);
+  }
+  const int kt_first = (k_lo / AT_KEYS) * AT_KEYS;
+  const int n_blocks = (k_hi - kt_first) / AT_KEYS + 1;
+  u32x4 kreg[KCH], vreg[VCH];
+  int kpg[KCH], vpg[VCH];
+  const int pmask = (1 << page_shift) - 1;
+  auto load_pages = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j;
+      const int kabs = kt + c / (DK16 * 2);
+      kpg[j] = (c < AT_KEYS * DK16 * 2 && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+    }
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + 256 * j;
+      const int kabs = kt + c / VPC;
+      vpg[j] = (c < AT_KEYS * VPC && (c % VPC) * 8 < dv && kabs >= k_lo && kabs <= k_hi) ? tbl[kabs >> page_shift] : -1;
+    }
+  };
+  auto load_block = [&](int kt) {
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j;
+      const int key = c / (DK16 * 2), pc = c % (DK16 * 2);
+      kreg[j] = u32x4{0u, 0u, 0u, 0u};
+      if (kpg[j] >= 0)
+        kreg[j] = *(const u32x4*)(kc + ((((size_t)kpg[j] * k_slots + ks_) << page_shift) + ((kt + key) & pmask)) * DK + pc * 8);
+    }
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + 256 * j;
+      const int key = c / VPC, pc = c % VPC;
+      vreg[j] = u32x4{0u, 0u, 0u, 0u};
+      if (vpg[j] >= 0)
+        vreg[j] = *(const u32x4*)(vc + ((((size_t)vpg[j] * v_heads + vh) << page_shift) + ((kt + key) & pmask)) * dv + pc * 8);
+    }
+  };
+  auto store_block = [&](int buf) {
+    bf16_t* kd = Ks + buf * KSZ;
+    bf16_t* vd = Vs + buf * VSZ;
+#pragma unroll
+    for (int j = 0; j < KCH; ++j) {
+      const int c = tid + 256 * j;
+      if (c >= AT_KEYS * DK16 * 2) continue;
+      *(u32x4*)(kd + (size_t)(c / (DK16 * 2)) * KLD + (c % (DK16 * 2)) * 8) = kreg[j];
+    }
+#pragma unroll
+    for (int j = 0; j < VCH; ++j) {
+      const int c = tid + 256 * j;
+      if (c >= AT_KEYS * VPC) continue;
+      *(u32x4*)(vd + (size_t)(c / VPC) * VLD + (c % VPC) * 8) = vreg[j];
+    }
+  };
+  // what this lane names in a transposing load of V: key 4 half + (lane % 16) / 4, dims 16 ((lane / 16) % 2) + 4 (lane % 4)
+  const int v_lane = (half * 4 + ((lane & 15) >> 2)) * VLD + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+  floatx16 o[DB];
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) o[db][e] = 0.f;
+  float m = -INFINITY, l = 0.f;
+  const float log2e = 1.4426950408889634f;
+  const float sl = softcap > 0.f ? log2e : scale * log2e;  // capped scores are final; raw ones are scaled in the exponent
+  const float cap_in = softcap > 0.f ? 2.0f * log2e * scale / softcap : 0.f;
+  load_pages(kt_first);
+  load_block(kt_first);
+  load_pages(kt_first + AT_KEYS);
+  store_block(0);
+  __syncthreads();
+  int buf = 0;
+  for (int it = 0, kt = kt_first; it < n_blocks; ++it, kt += AT_KEYS, buf ^= 1) {
+    const bool more = it + 1 < n_blocks;
+    if (more) {
+      load_block(kt + AT_KEYS);
+      load_pages(kt + 2 * AT_KEYS);
+    }
+    if (wave_on && kt <= wave_hi) {
+      const bf16_t* Kb = Ks + buf * KSZ;
+      const bf16_t* Vb = Vs + buf * VSZ + v_lane;
+      floatx16 sc[2];
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e) sc[kb][e] = 0.f;
+        const bf16_t* kr = Kb + (size_t)(kb * 32 + qi) * KLD + half * 8;
+#pragma unroll
+        for (int i = 0; i < DK16; ++i) sc[kb] = mfma32(*(const u32x4*)(kr + i * 16), qf[i], sc[kb]);
+      }
+      if (softcap > 0.f) {  // cap * tanh(x), tanh(x) = 1 - 2 / (1 + exp(2x))
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            sc[kb][e] = softcap * (1.0f - 2.0f * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(sc[kb][e] * cap_in)));
+      }
+      const bool all_visible = kt + AT_KEYS - 1 <= wave_lo_pos && kt >= wave_first;
+      if (!all_visible) {
+        const int key0 = kt + half * 4;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            const int key = key0 + kb * 32 + 8 * (e >> 2) + (e & 3);
+            sc[kb][e] = (key >= first_q && key <= pos_q) ? sc[kb][e] : -INFINITY;
+          }
+      }
+      // the maximum of the scores as they enter the exponent (a negative scale turns the order round)
+      float mx = -INFINITY;
+#pragma unroll
+      for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) mx = fmaxf(mx, sc[kb][e] * sl);
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = (mx > m + 8.0f) ? mx : m;  // moves only when it grows by more than 2^8
+      u32x4 pb[2][2];
+      if (m_new == -INFINITY) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int st = 0; st < 2; ++st) pb[kb][st] = u32x4{0u, 0u, 0u, 0u};
+      } else {
+        float rs = 0.f;
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb) {
+          float p[16];
+#pragma unroll
+          for (int e = 0; e < 16; ++e) {
+            p[e] = __builtin_amdgcn_exp2f(fmaf(sc[kb][e], sl, -m_new));
+            rs += p[e];
+          }
+#pragma unroll
+          for (int st = 0; st < 2; ++st)
+            pb[kb][st] = u32x4{pack_bf16(p[8 * st], p[8 * st + 1]), pack_bf16(p[8 * st + 2], p[8 * st + 3]),
+                               pack_bf16(p[8 * st + 4], p[8 * st + 5]), pack_bf16(p[8 * st + 6], p[8 * st + 7])};
+        }
+        rs += __shfl_xor(rs, 32, 64);
+        if (m_new != m) {
+          const float alpha = __builtin_amdgcn_exp2f(m - m_new);
+          l *= alpha;
+#pragma unroll
+          for (int db = 0; db < DB; ++db)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) o[db][e] *= alpha;
+          m = m_new;
+        }
+        l += rs;
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            const int k0 = kb * 32 + 16 * st;
+            const u32x2 lo = lds_read_tr16(Vb + k0 * VLD + db * 32);
+            const u32x2 hi = lds_read_tr16(Vb + (k0 + 8) * VLD + db * 32);
+            o[db] = mfma32(u32x4{lo.x, lo.y, hi.x, hi.y}, pb[kb][st], o[db]);
+          }
+      }
+    }
+    if (more) store_block(buf ^ 1);
+    __syncthreads();
+  }
+  if (!wave_on || wq >= nrows) return;
+  const float inv = 1.0f / l;
+  float* orow = out + (size_t)(row0 + wq) * ldo + (size_t)s * dv;
+#pragma unroll
+  for (int db = 0; db < DB; ++db)
+#pragma unroll
+    for (int e4 = 0; e4 < 4; ++e4) {
+      const int d = db * 32 + 8 * e4 + half * 4;
+      if (d < dv) *(float4*)(orow + d) = float4{o[db][4 * e4] * inv, o[db][4 * e4 + 1] * inv, o[db][4 * e4 + 2] * inv, o[db][4 * e4 + 3] * inv};
+    }
+}
+
+template <int DK16, int DB>
+static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq, float* out, int ldo, const bf16_t* kc,
+                        const bf16_t* vc, const int* block_table, int max_blocks, const int* tiles, const int* positions, int maps,
+                        int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window, float scale, float softcap) {
+  const size_t smem = (size_t)2 * AT_KEYS * ((DK16 * 16 + 8) + (DB * 32 + 32)) * sizeof(bf16_t);
+  static bool raised = false;
+  if (smem > 64 * 1024 && !raised) {
+    if (hipFuncSetAttribute((const void*)attention_dv_tiles_kernel<DK16, DB>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem) != hipSuccess)
+      return -1;
+    raised = true;
+  }
+  attention_dv_tiles_kernel<DK16, DB><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, block_table, max_blocks, tiles, positions,
+                                                                 maps, per_kv, k_slots, v_heads, dv, page_shift, window, scale, softcap);
+  return 0;
+}
+
+// Returns 1 (declined) for sizes it does not take: dk a multiple of 16 up to 256, dv a multiple of 8 up to 256, bf16.
+extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ldo, const void* kcache, const void* vcache,
+                                      const int* block_table, int max_blocks, const int* tiles, int n_tiles,
+                                      const int* positions, int heads, int kv_heads, int maps, int dk, int dv, int page_size,
+                                      int window, float scale, float softcap, hipStream_t stream) {
+  if (n_tiles <= 0) return 0;
+  if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || maps <= 0) JLLM_FAIL("attention: %d query heads over %d kv heads with %d maps", heads, kv_heads, maps);
+  if ((dk & 15) || dk < 16 || dk > 256 || (dv & 7) || dv < 8 || dv > 256) return 1;
+  if (!(scale > 0.f) || softcap < 0.f) return 1;  // the maximum is taken before the scale's sign could matter
+  if ((ldq & 7) || (ldo & 3) || ((uintptr_t)q & 15) || ((uintptr_t)out & 15) || ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15)) return 1;
+  if (page_size <= 0 || (page_size & (page_size - 1)) || n_tiles > 65535 || heads * maps > 65535) return 1;
+  int page_shift = 0;
+  while ((1 << page_shift) < page_size) ++page_shift;
+  const int q_slots = heads * maps, per_kv = maps * (heads / kv_heads);
+  dim3 grid(q_slots, n_tiles);
+  const int db = (dv + 31) / 32;
+  int rc = 1;
+#define AT_ARGS grid, stream, (const bf16_t*)q, ldq, out, ldo, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, max_blocks, \
+                tiles, positions, maps, per_kv, kv_heads * maps, kv_heads, dv, page_shift, window, scale, softcap
+#define AT_DB(N)                                  \
+  switch (db) {                                   \
+    case 1: rc = launch_tiles<N, 1>(AT_ARGS); break; \
+    case 2: rc = launch_tiles<N, 2>(AT_ARGS); break; \
+    case 3: rc = launch_tiles<N, 3>(AT_ARGS); break; \
+    case 4: rc = launch_tiles<N, 4>(AT_ARGS); break; \
+    case 8: rc = launch_tiles<N, 8>(AT_ARGS); break; \
+    default: return 1;                            \
+  }
+  switch (dk / 16) {
+    case 1: AT_DB(1) break;
+    case 2: AT_DB(2) break;
+    case 3: AT_DB(3) break;
+    case 4: AT_DB(4) break;
+    case 6: AT_DB(6) break;
+    case 8: AT_DB(8) break;
+    case 16: AT_DB(16) break;
+    default: return 1;
+  }
+#undef AT_DB
+#undef AT_ARGS
+  if (rc < 0) JLLM_FAIL("attention: cannot reserve LDS");
+  JLLM_CHECK_LAUNCH("attention_dv_bf16");
+  return 0;
+}

@@ -6,18 +6,23 @@
 //   short_conv_silu      y[t, c] = silu(sum_j taps[c, K - 1 - j] x[t - j, c]); inputs before the step's first row of a
 //                        request come from that request's state, inputs before position 0 are the state's zeros
 //   short_conv_advance   the state's K - 1 inputs per channel move on by the request's rows of this step
-//   gated_delta          per (request, head), token by token, with S [dk, dv] in registers:
+//   gated_delta          token by token, with S [dk, dv] in registers:
 //                          q <- q / sqrt(sum q^2 + 1e-6) / sqrt(dk), k <- k / sqrt(sum k^2 + 1e-6)
 //                          beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias))
 //                          S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
-//                        computed as  S^T k and S^T q of the old S in one pass, o = g S^T q + (k . q) u
-//                          out = o / sqrt(mean(o^2) + eps) * gain * silu(gate)
+//                        computed as  S^T k and S^T q of the old S in one pass, o = g S^T q + (k . q) u.
+//                        The columns of S never meet: column j only needs v[j], so a workgroup is ONE wave that owns 16
+//                        value columns of one head of one request (4 lanes per column, a quarter of the key rows
+//                        each) and walks the request's rows without a barrier; a step of one request and 16 heads of
+//                        128 x 128 is 128 such waves. The read-out o goes out raw in fp32; the heads' norm, gain and
+//                        gate need all columns of a head and are the finishing kernel's (attention_dv.hip).
 #include <math.h>
 
 #include "common.h"
 
 #define CONV_MAX_TAPS 16
-#define GDR_MAX_PARTS 32
+#define GDR_COLS 16   // value columns of a wave
+#define GDR_PARTS 4   // lanes per column: each owns a quarter of the key rows
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
@@ -112,159 +117,124 @@ extern "C" int jllm_short_conv(const void* x, int ldx, void* y, int ldy, int dty
 struct GdrArgs {
   const void* qkv;   // [rows, ldc]: q (kv_heads x dk) | k (kv_heads x dk) | v (heads x dv), convolved
   int ldc;
-  const void* proj;  // [rows, ldp]: the projection's row, which holds the gate (heads x dv), a and b (heads each)
-  int ldp, gate_off, a_off, b_off;
+  const void* proj;  // [rows, ldp]: the projection's row, which holds a and b (heads each) at their offsets
+  int ldp, a_off, b_off;
   const void* a_log;    // [heads]
   const void* dt_bias;  // [heads]
-  const void* gain;     // [dv]
   float* state;         // [slots, heads, dk, dv]
-  void* out;            // [rows, ldo]: heads x dv
+  float* out;           // [rows, ldo]: heads x dv, the raw read-out
   int ldo;
   const int* row_req;
   const int* state_slots;
-  int n_rows, heads, kv_heads, dk, dv, parts;
-  float eps;
+  int n_rows, heads, kv_heads, dk, dv;
 };
 
-// Threads (j, part): j = tid % dv is a value column, part = tid / dv owns rows part, part + P, ... of S (E at most).
-// The workgroup is filled up to whole waves; the threads beyond dv * P only take part in the waves' sums.
-template <typename T, typename TW, int E>
-__global__ void gated_delta_kernel(GdrArgs A) {
-  extern __shared__ float sm[];
-  const int dk = A.dk, dv = A.dv, P = A.parts;
-  const int nthreads = blockDim.x;
-  const int tid = threadIdx.x;
-  const int j = tid % dv, part = tid / dv;
-  const bool act = part < P;
-  const int lane = tid & 63;
-  // per parity: q[dk], k[dk], partial sums [2][P][dv], o[dv]
-  const int per = 2 * dk + 2 * P * dv + dv;
+// what a lane needs of one row: its quarter of q and k, its column's v, the head's a and b
+template <typename T, int E>
+struct GdrRow {
+  float q[E], k[E], v, a, b;
+  __device__ __forceinline__ void load(const GdrArgs& A, size_t row, int kvh, int h, int i0, int col, bool col_on) {
+    const T* cr = (const T*)A.qkv + row * A.ldc;
+    const T* qr = cr + (size_t)kvh * A.dk;
+    const T* kr = cr + (size_t)(A.kv_heads + kvh) * A.dk;
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+      const bool on = i0 + e < A.dk;
+      q[e] = on ? ldf(qr, i0 + e) : 0.f;
+      k[e] = on ? ldf(kr, i0 + e) : 0.f;
+    }
+    v = col_on ? ldf(cr, (size_t)2 * A.kv_heads * A.dk + (size_t)h * A.dv + col) : 0.f;
+    const T* pr = (const T*)A.proj + row * A.ldp;
+    a = ldf(pr, A.a_off + h);
+    b = ldf(pr, A.b_off + h);
+  }
+};
+
+__device__ __forceinline__ float parts_sum(float v) {  // over the four lanes of a column, the same in all of them
+  v += __shfl_xor(v, 16, 64);
+  v += __shfl_xor(v, 32, 64);
+  return v;
+}
+
+// lane = part * 16 + c: column blockIdx.z * 16 + c, key rows part * E .. + E
+template <typename T, typename TW, int E, bool AHEAD>
+__global__ __launch_bounds__(64) void gated_delta_kernel(GdrArgs A) {
+  const int lane = threadIdx.x;
+  const int c = lane & (GDR_COLS - 1), part = lane / GDR_COLS;
   const int req = blockIdx.x, h = blockIdx.y;
+  const int col = blockIdx.z * GDR_COLS + c;
+  const bool col_on = col < A.dv;
   int lo, n;
   rows_of_request(A.row_req, A.n_rows, req, lo, n);
   if (n == 0) return;
   const int kvh = h / (A.heads / A.kv_heads);
-  float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * dk * dv;
+  const int i0 = part * E;
+  float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * A.dk * A.dv;
   float S[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const int i = part + e * P;
-    S[e] = (act && i < dk) ? S_at[(size_t)i * dv + j] : 0.f;
-  }
+  for (int e = 0; e < E; ++e) S[e] = (col_on && i0 + e < A.dk) ? S_at[(size_t)(i0 + e) * A.dv + col] : 0.f;
   const float decay_rate = expf(ldf((const TW*)A.a_log, h));
   const float dtb = ldf((const TW*)A.dt_bias, h);
-  const float gain = ldf((const TW*)A.gain, j);
-  const float q_scale = 1.0f / sqrtf((float)dk);
-  const T* conv = (const T*)A.qkv;
-  const T* proj = (const T*)A.proj;
-  T* out = (T*)A.out;
+  const float q_scale = 1.0f / sqrtf((float)A.dk);
+  GdrRow<T, E> cur, nxt;
+  cur.load(A, (size_t)lo, kvh, h, i0, col, col_on);
   for (int r = 0; r < n; ++r) {
-    const size_t row = (size_t)(lo + r);
-    float* buf = sm + (size_t)(r & 1) * per;
-    float* qs = buf;
-    float* ks = buf + dk;
-    float* pk = buf + 2 * dk;
-    float* pq = pk + P * dv;
-    float* os = pq + P * dv;
-    const T* cr = conv + row * A.ldc;
-    for (int i = tid; i < 2 * dk; i += nthreads)
-      buf[i] = ldf(cr, (size_t)(i < dk ? 0 : A.kv_heads * dk) + (size_t)kvh * dk + (i < dk ? i : i - dk));
-    const float v = ldf(cr, (size_t)2 * A.kv_heads * dk + (size_t)h * dv + j);
-    const T* pr = proj + row * A.ldp;
-    const float a = ldf(pr, A.a_off + h), b = ldf(pr, A.b_off + h);
-    const float gate = ldf(pr, (size_t)A.gate_off + (size_t)h * dv + j);
-    __syncthreads();
-    // every wave sums the squares and q . k for itself, in the same order
-    float sq = 0.f, sk = 0.f, qk = 0.f;
-    for (int i = lane; i < dk; i += 64) {
-      sq = fmaf(qs[i], qs[i], sq);
-      sk = fmaf(ks[i], ks[i], sk);
-      qk = fmaf(qs[i], ks[i], qk);
-    }
-    sq = wave_sum(sq), sk = wave_sum(sk), qk = wave_sum(qk);
-    const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
-    qk *= rq * rk;
-    float dk_ = 0.f, dq_ = 0.f;
+    if (AHEAD && r + 1 < n) nxt.load(A, (size_t)(lo + r + 1), kvh, h, i0, col, col_on);  // in flight under this row's sums
+    float sq = 0.f, sk = 0.f, qk = 0.f, dk_ = 0.f, dq_ = 0.f;
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-      const int i = part + e * P;
-      if (i < dk) {
-        dk_ = fmaf(S[e], ks[i], dk_);
-        dq_ = fmaf(S[e], qs[i], dq_);
-      }
+      sq = fmaf(cur.q[e], cur.q[e], sq);
+      sk = fmaf(cur.k[e], cur.k[e], sk);
+      qk = fmaf(cur.q[e], cur.k[e], qk);
+      dk_ = fmaf(S[e], cur.k[e], dk_);
+      dq_ = fmaf(S[e], cur.q[e], dq_);
     }
-    if (act) {
-      pk[part * dv + j] = dk_;
-      pq[part * dv + j] = dq_;
-    }
-    __syncthreads();
-    float Sk = 0.f, Sq = 0.f;
-    for (int p = 0; p < P; ++p) {
-      Sk += pk[p * dv + j];
-      Sq += pq[p * dv + j];
-    }
-    Sk *= rk, Sq *= rq;
-    const float z = a + dtb;
+    sq = parts_sum(sq), sk = parts_sum(sk), qk = parts_sum(qk), dk_ = parts_sum(dk_), dq_ = parts_sum(dq_);
+    const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+    const float z = cur.a + dtb;
     const float sp = z > 20.f ? z : log1pf(expf(z));
     const float g = expf(-decay_rate * sp);
-    const float beta = 1.0f / (1.0f + expf(-b));
-    const float u = beta * (v - g * Sk);
-    const float o = fmaf(g, Sq, qk * u);
+    const float beta = 1.0f / (1.0f + expf(-cur.b));
+    const float u = beta * (cur.v - g * (dk_ * rk));
+    const float o = fmaf(g, dq_ * rq, qk * rq * rk * u);
     const float ku = u * rk;
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const int i = part + e * P;
-      if (i < dk) S[e] = fmaf(ks[i], ku, g * S[e]);
-    }
-    if (part == 0) os[j] = o;
-    __syncthreads();
-    float ss = 0.f;
-    for (int i = lane; i < dv; i += 64) ss = fmaf(os[i], os[i], ss);
-    ss = wave_sum(ss);
-    if (part == 0) {
-      stf(out + row * A.ldo, (size_t)h * dv + j, o * norm_scale(ss, dv, A.eps) * gain * silu_f(gate));
-    }
+    for (int e = 0; e < E; ++e) S[e] = fmaf(cur.k[e], ku, g * S[e]);
+    if (part == 0 && col_on) A.out[(size_t)(lo + r) * A.ldo + (size_t)h * A.dv + col] = o;
+    if (AHEAD)
+      cur = nxt;
+    else if (r + 1 < n)
+      cur.load(A, (size_t)(lo + r + 1), kvh, h, i0, col, col_on);
   }
 #pragma unroll
-  for (int e = 0; e < E; ++e) {
-    const int i = part + e * P;
-    if (act && i < dk) S_at[(size_t)i * dv + j] = S[e];
-  }
+  for (int e = 0; e < E; ++e)
+    if (col_on && i0 + e < A.dk) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
 }
 
-extern "C" int jllm_gated_delta(const void* qkv, int ldc, const void* proj, int ldp, int gate_off, int a_off, int b_off,
-                                int dtype, const void* a_log, const void* dt_bias, const void* gain, int w_dtype, float* state,
-                                void* out, int ldo, const int* row_req, const int* state_slots, int n_rows, int n_requests,
-                                int heads, int kv_heads, int dk, int dv, float eps, hipStream_t stream) {
+extern "C" int jllm_gated_delta(const void* qkv, int ldc, const void* proj, int ldp, int a_off, int b_off, int dtype,
+                                const void* a_log, const void* dt_bias, int w_dtype, float* state, float* out, int ldo,
+                                const int* row_req, const int* state_slots, int n_rows, int n_requests, int heads,
+                                int kv_heads, int dk, int dv, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 65535) JLLM_FAIL("gated_delta: %d heads over %d key heads", heads, kv_heads);
-  if (dk <= 0 || dv <= 0 || dv > 1024) JLLM_FAIL("gated_delta: key size %d, value size %d (values up to 1024 are taken)", dk, dv);
+  if (dk <= 0 || dk > GDR_PARTS * 64 || dv <= 0 || dv > GDR_COLS * 65535) JLLM_FAIL("gated_delta: key size %d (1..%d are taken), value size %d", dk, GDR_PARTS * 64, dv);
   if (n_requests <= 0 || n_requests > n_rows) JLLM_FAIL("gated_delta: %d requests in %d rows", n_requests, n_rows);
-  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || ldp < gate_off + heads * dv || ldp < a_off + heads || ldp < b_off + heads)
+  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || ldp < a_off + heads || ldp < b_off + heads || a_off < 0 || b_off < 0)
     JLLM_FAIL("gated_delta: short rows");
-  // as many parts of the key rows as keep a workgroup near 256 threads; more where a thread would hold too many
-  int parts = 1;
-  while (parts * 2 * dv <= 256 && parts * 2 <= dk && parts < GDR_MAX_PARTS) parts *= 2;
-  while ((dk + parts - 1) / parts > 64 && parts * 2 * dv <= 1024 && parts < GDR_MAX_PARTS) parts *= 2;
-  const int per_thread = (dk + parts - 1) / parts;
-  if (per_thread > 64) JLLM_FAIL("gated_delta: a state of %d x %d per head does not fit a workgroup's registers", dk, dv);
-  GdrArgs A{qkv, ldc, proj, ldp, gate_off, a_off, b_off, a_log, dt_bias, gain, state, out, ldo, row_req, state_slots,
-            n_rows, heads, kv_heads, dk, dv, parts, eps};
-  const size_t smem = (size_t)2 * (2 * dk + 2 * parts * dv + dv) * sizeof(float);
-  if (smem > 64 * 1024) JLLM_FAIL("gated_delta: %zu bytes of LDS for key size %d, value size %d", smem, dk, dv);
-  dim3 grid(n_requests, heads);
-  const int threads = (dv * parts + 63) / 64 * 64;
-#define GDR_LAUNCH(E) gated_delta_kernel<T, TW, E><<<grid, threads, smem, stream>>>(A)
+  GdrArgs A{qkv, ldc, proj, ldp, a_off, b_off, a_log, dt_bias, state, out, ldo, row_req, state_slots, n_rows, heads, kv_heads, dk, dv};
+  dim3 grid(n_requests, heads, (dv + GDR_COLS - 1) / GDR_COLS);
+  const int per_lane = (dk + GDR_PARTS - 1) / GDR_PARTS;
+#define GDR_LAUNCH(E, AHEAD) gated_delta_kernel<T, TW, E, AHEAD><<<grid, 64, 0, stream>>>(A)
   JLLM_DISPATCH_1(dtype, T, {
     JLLM_DISPATCH_1(w_dtype, TW, {
-      if (per_thread <= 8)
-        GDR_LAUNCH(8);
-      else if (per_thread <= 16)
-        GDR_LAUNCH(16);
-      else if (per_thread <= 32)
-        GDR_LAUNCH(32);
+      if (per_lane <= 8)
+        GDR_LAUNCH(8, true);
+      else if (per_lane <= 16)
+        GDR_LAUNCH(16, true);
+      else if (per_lane <= 32)
+        GDR_LAUNCH(32, true);
       else
-        GDR_LAUNCH(64);
+        GDR_LAUNCH(64, false);
     })
   })
 #undef GDR_LAUNCH

@@ -78,9 +78,9 @@ def _declare(lib) -> None:
         "jllm_layernorm_seam": [_P, _P, _I, _I, _P, _I, _P, _I, _I, _F, _F, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _P],
         "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
         "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
-        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _P, _I, _I, _P],
+        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _P, _I, _I, _P],
         "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
-        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _I, _P, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P],
+        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -113,6 +113,7 @@ _OPTIONAL_SIGS = {
     "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_gemm_mfma_grouped_bf16": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _I, _P],
+    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -1142,15 +1143,34 @@ def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     return out
 
 
-_fast_attention_dv = None
+WIDE_TILE_ROWS = 128  # rows of one request per tile of the matrix-core kernel (csrc/attention_dv_mfma.hip)
+
+
+def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, maps, dk, dv, scale,
+                       softcap, window, meta) -> bool:
+    """The matrix-core kernel: bf16 pages, fp32 out, and the step's rows cut into tiles by the caller (``meta``:
+    "tiles_dev" int32 [n_tiles, 4] as (request, first row, rows, first position or -1), "n_tiles")."""
+    tiles = meta.get("tiles_dev") if meta else None
+    if tiles is None or q.dtype != torch.bfloat16 or out.dtype != torch.float32:
+        return False
+    n_tiles = int(meta["n_tiles"])
+    _i32(tiles, 4 * n_tiles, "tiles")
+    return _try("jllm_attention_dv_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+                _ptr(block_table), block_table.shape[1], _ptr(tiles), n_tiles, _ptr(positions), heads, kv_heads, maps, dk, dv,
+                k_cache.shape[2], int(window), float(scale), float(softcap), _stream())
+
+
+HEAD_GATES = {"sigmoid": 0, "silu": 1}
 
 
 def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: torch.dtype, *, lam: float = 0.0,
                  normed: bool = False, eps: float = 0.0, norm_mul: float = 1.0, gain: Optional[torch.Tensor] = None,
-                 gate: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """From the attention's rows [T, heads x maps x dv] to the output product's input [T, heads x dv]: with two maps
+                 gate: Optional[torch.Tensor] = None, gate_fn: str = "sigmoid") -> torch.Tensor:
+    """From a mixer's heads [T, heads x maps x dv] to the output product's input [T, heads x dv]: with two maps
     o = a1 - lam * a2; ``normed``: o / sqrt(mean(o^2) + eps) * norm_mul per head (times ``gain`` [dv]); with ``gate``
-    ([T, heads x dv], a view with any row stride) times sigmoid(gate)."""
+    ([T, heads x dv], a view with any row stride) times sigmoid(gate) or, ``gate_fn`` "silu", silu(gate)."""
+    if gate_fn not in HEAD_GATES:
+        raise KernelError(f"heads_finish: gate function '{gate_fn}' ({sorted(HEAD_GATES)} are built)")
     _dev(att, gain, gate)
     _rows2d(att, "attention rows")
     T = att.shape[0]
@@ -1167,8 +1187,8 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
         return out
     _call("jllm_heads_finish", _ptr(att), att.stride(0), _code(att.dtype), T, heads, maps, dv, float(lam), 1 if normed else 0,
           float(eps), float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
-          gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, _ptr(out),
-          out.stride(0), _code(out.dtype), _stream())
+          gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, HEAD_GATES[gate_fn],
+          _ptr(out), out.stride(0), _code(out.dtype), _stream())
     return out
 
 
@@ -1179,21 +1199,14 @@ MAX_CONV_TAPS = 16
 
 
 def check_gated_delta_shape(heads: int, kv_heads: int, dk: int, dv: int, taps: int) -> None:
-    """Raises when the delta-rule kernels do not take these sizes (asked when a model is built): a head's state of
-    dk x dv fp32 numbers lives in the registers of one workgroup."""
+    """Raises when the delta-rule kernels do not take these sizes (asked when a model is built): a wave keeps a
+    quarter of the key rows of 16 value columns per lane."""
     if heads <= 0 or kv_heads <= 0 or heads % kv_heads != 0:
         raise KernelError(f"gated delta rule: {heads} heads over {kv_heads} key heads")
     if not 1 <= taps <= MAX_CONV_TAPS:
         raise KernelError(f"gated delta rule: a convolution of {taps} taps (1..{MAX_CONV_TAPS} are taken)")
-    if dk <= 0 or not 0 < dv <= 1024:
-        raise KernelError(f"gated delta rule: key size {dk}, value size {dv}")
-    parts = 1
-    while parts * 2 * dv <= 256 and parts * 2 <= dk and parts < 32:
-        parts *= 2
-    while -(-dk // parts) > 64 and parts * 2 * dv <= 1024 and parts < 32:
-        parts *= 2
-    if -(-dk // parts) > 64 or 2 * (2 * dk + 2 * parts * dv + dv) * 4 > 64 * 1024:
-        raise KernelError(f"gated delta rule: a state of {dk} x {dv} per head does not fit a workgroup")
+    if not 0 < dk <= 256 or dv <= 0:
+        raise KernelError(f"gated delta rule: key size {dk} (1..256 are taken), value size {dv}")
 
 
 def short_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor,
@@ -1222,17 +1235,15 @@ def short_conv(x: torch.Tensor, taps: torch.Tensor, state: torch.Tensor, row_req
     return y
 
 
-def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, gate_off: int, a_off: int, b_off: int, a_log: torch.Tensor,
-                dt_bias: torch.Tensor, gain: torch.Tensor, state: torch.Tensor, row_req: torch.Tensor,
-                state_slots: torch.Tensor, n_requests: int, heads: int, kv_heads: int, dk: int, dv: int,
-                eps: float) -> torch.Tensor:
+def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a_log: torch.Tensor, dt_bias: torch.Tensor,
+                state: torch.Tensor, row_req: torch.Tensor, state_slots: torch.Tensor, n_requests: int, heads: int,
+                kv_heads: int, dk: int, dv: int) -> torch.Tensor:
     """The gated delta rule over the step's rows, request by request and token by token, from and into ``state``
     [slots, heads, dk, dv] (fp32). ``qkv`` [T, kv_heads x dk | kv_heads x dk | heads x dv] are the convolved q, k, v;
-    ``proj`` rows hold, at the given offsets, the output gate (heads x dv) and the inputs a and b of decay and write
-    strength (heads each). Per head: q and k become unit vectors (q also / sqrt(dk)); beta = sigmoid(b); g = exp(-exp(
-    a_log) softplus(a + dt_bias)); S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q; the result is o / sqrt(
-    mean(o^2) + eps) * gain * silu(gate), [T, heads x dv]."""
-    _dev(qkv, proj, a_log, dt_bias, gain, state, row_req, state_slots)
+    ``proj`` rows hold, at the given offsets, the inputs a and b of decay and write strength (heads each). Per head:
+    q and k become unit vectors (q also / sqrt(dk)); beta = sigmoid(b); g = exp(-exp(a_log) softplus(a + dt_bias));
+    S <- g S; u = beta (v - S^T k); S <- S + k u^T; o = S^T q. Returns the raw o, fp32 [T, heads x dv]."""
+    _dev(qkv, proj, a_log, dt_bias, state, row_req, state_slots)
     _rows2d(qkv, "convolved q, k, v")
     _rows2d(proj, "projection rows")
     T = qkv.shape[0]
@@ -1240,23 +1251,22 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, gate_off: int, a_off: int
         raise KernelError("the projection rows and the convolved rows must agree in rows and type")
     if qkv.shape[1] != 2 * kv_heads * dk + heads * dv:
         raise KernelError(f"convolved rows have {qkv.shape[1]} entries, expected {2 * kv_heads * dk + heads * dv}")
-    if max(gate_off + heads * dv, a_off + heads, b_off + heads) > proj.shape[1] or min(gate_off, a_off, b_off) < 0:
-        raise KernelError("gate, a or b lie outside the projection rows")
-    if a_log.numel() != heads or dt_bias.numel() != heads or gain.numel() != dv:
-        raise KernelError(f"a_log and dt_bias must have {heads} entries, the gain {dv}")
-    wd = _same_type("a_log, dt_bias and the gain", a_log, dt_bias, gain)
+    if max(a_off + heads, b_off + heads) > proj.shape[1] or min(a_off, b_off) < 0:
+        raise KernelError("a or b lie outside the projection rows")
+    if a_log.numel() != heads or dt_bias.numel() != heads:
+        raise KernelError(f"a_log and dt_bias must have {heads} entries")
+    wd = _same_type("a_log and dt_bias", a_log, dt_bias)
     if state.dtype != torch.float32 or not state.is_contiguous() or state.dim() != 4 or state.shape[1:] != (heads, dk, dv):
         raise KernelError(f"the state must be a contiguous fp32 [slots, {heads}, {dk}, {dv}] tensor")
     _i32(row_req, T, "row -> request map")
     _i32(state_slots, n_requests, "state slots")
-    out = activation_rows(T, heads * dv, qkv.dtype, qkv.device)
+    out = torch.empty((T, heads * dv), dtype=torch.float32, device=qkv.device)
     if T == 0:
         return out
-    _call("jllm_gated_delta", _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(gate_off), int(a_off), int(b_off),
-          _code(qkv.dtype), _ptr(a_log), _ptr(dt_bias), _ptr(gain), wd, _ptr(state), _ptr(out), out.stride(0), _ptr(row_req),
-          _ptr(state_slots), T, int(n_requests), heads, kv_heads, dk, dv, float(eps), _stream())
+    _call("jllm_gated_delta", _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(a_off), int(b_off), _code(qkv.dtype),
+          _ptr(a_log), _ptr(dt_bias), wd, _ptr(state), _ptr(out), out.stride(0), _ptr(row_req), _ptr(state_slots), T,
+          int(n_requests), heads, kv_heads, dk, dv, _stream())
     return out
-
 
 
 MOE_TILE_ROWS = 16      # rows of one expert that a workgroup of the grouped products takes in steps of few rows ...

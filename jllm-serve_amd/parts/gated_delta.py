@@ -8,9 +8,10 @@ request), so nothing grows with the context and nothing is paged.
 A step is
   1. one product with the stacked weight [W_q | W_k | W_v | W_g | W_a | W_b],
   2. the convolutions with silu over the first columns, reading and advancing their state (``ops.short_conv``),
-  3. the recurrence over each request's rows in order, with unit norms, decay, write strength, the heads' norm and
-     the output gate inside (``ops.gated_delta``),
-  4. the output product.
+  3. the recurrence over each request's rows in order, with unit norms, decay and write strength inside
+     (``ops.gated_delta``; its value columns are spread over workgroups, so its read-out comes back raw),
+  4. the heads' norm, gain and silu gate (``ops.heads_finish``, the kernel that ends attention heads too),
+  5. the output product.
 The same launches serve portions of prompts and single rows: the recurrence visits a request's rows one after the
 other either way, so its result does not depend on how a prompt was cut.
 """
@@ -65,10 +66,11 @@ class GatedDelta(Part):
         taps = [get(self._name(n, nm.conv_suffix)) for n in "qkv"]
         dt = taps[0].dtype if all(t.dtype == taps[0].dtype for t in taps) else torch.float32
         self.taps = torch.cat([t.to(dt) for t in taps], dim=0).contiguous()
-        small = [get(self._name(n)) for n in ("a_log", "dt_bias", "norm")]
-        if any(t.dtype != small[0].dtype for t in small):
+        small = [get(self._name(n)) for n in ("a_log", "dt_bias")]
+        if small[0].dtype != small[1].dtype:
             small = [t.float() for t in small]
-        self.a_log, self.dt_bias, self.gain = small
+        self.a_log, self.dt_bias = small
+        self.gain = get(self._name("norm"))
         self.w_o = get(self._name("o"))
 
     def state_spec(self):
@@ -82,8 +84,10 @@ class GatedDelta(Part):
         matrix, tail = slot.state
         y = ops.gemm(xb, self.w_in, out_dtype=self.build.dtype, exact=self.build.exact)
         qkv = ops.short_conv(y, self.taps, tail, step.row_req, step.state_slots, step.n_requests)
-        return ops.gated_delta(qkv, y, self.gate_at, self.a_at, self.b_at, self.a_log, self.dt_bias, self.gain, matrix,
-                               step.row_req, step.state_slots, step.n_requests, s.heads, s.kv_heads, s.dim, s.vdim, s.eps)
+        o = ops.gated_delta(qkv, y, self.a_at, self.b_at, self.a_log, self.dt_bias, matrix, step.row_req, step.state_slots,
+                            step.n_requests, s.heads, s.kv_heads, s.dim, s.vdim)
+        return ops.heads_finish(o, s.heads, 1, s.vdim, self.build.dtype, normed=True, eps=s.eps, gain=self.gain,
+                                gate=y[:, self.gate_at:self.gate_at + self.v_dim], gate_fn="silu")
 
     def output(self, xb, step, slot):
         return ops.gemm(self.heads_rows(xb, step, slot), self.w_o, out_dtype=torch.float32, exact=self.build.exact)

@@ -24,6 +24,25 @@ from ..weights.loader import WeightSpec
 from .base import BuildContext, Part, register_part
 
 
+class WideStepPlanner:
+    """What the matrix-core attention kernel wants to know about a batch, once per step for all such layers: every
+    request's rows cut into tiles of at most ``ops.WIDE_TILE_ROWS`` rows as (request, first row, rows, first position),
+    the tiles with the most keys first. A step of fixed size (every request one row) gets one tile per row in row order
+    with position -1: the kernel then reads the row's position on the device."""
+
+    key = ("wide_attention", ops.WIDE_TILE_ROWS)
+
+    def plan(self, batch):
+        from ..engine.step import StepPlan
+        R = ops.WIDE_TILE_ROWS
+        if batch.padded:
+            runs = [(r, r, 1, -1) for r in range(batch.rows)]
+        else:
+            runs = [(s.index, s.row0 + r, min(R, s.n - r), s.pos0 + r) for s in batch.segments for r in range(0, s.n, R)]
+            runs.sort(key=lambda t: -(t[3] + t[2]))
+        return StepPlan({"tiles": [v for t in runs for v in t]}, {"n_tiles": len(runs)})
+
+
 class WideAttention(Part):
     def __init__(self, spec: WideAttentionSpec, prefix: str, build: BuildContext, positions):
         if spec.maps not in (1, 2):
@@ -96,6 +115,19 @@ class WideAttention(Part):
         s = self.spec
         return PageSpec((CacheRow("k", (s.kv_heads * s.maps, s.dim), 1), CacheRow("v", (s.kv_heads, s.vdim), 1)), s.window)
 
+    def step_planners(self):
+        return [WideStepPlanner()]
+
+    @staticmethod
+    def _batch_facts(step):
+        meta = {"max_context": step.max_context, "requests": step.n_requests, "rows": step.n_tokens}
+        plan = step.plans.get(WideStepPlanner.key)
+        if plan is not None:
+            tiles = plan.arrays.get("tiles")
+            meta["n_tiles"] = plan.facts["n_tiles"]
+            meta["tiles_dev"] = tiles if tiles is not None and tiles.numel() else None
+        return meta
+
     def heads_rows(self, xb, step, slot):
         """The input of the output product, [rows, heads x vdim] in the run's type."""
         s, exact = self.spec, self.build.exact
@@ -106,7 +138,7 @@ class WideAttention(Part):
         ops.qkv_prepare(y, step.positions, g.slots if slot.writes else None, s.heads, s.kv_heads, s.maps, s.dim, s.vdim,
                         k_cache, v_cache, gq=self.g_q, gk=self.g_k, eps=s.eps, cos=cos, sin=sin, rot_dims=rdims,
                         temp_coef=s.q_temp_coef, temp_every=s.q_temp_every)
-        meta = {"max_context": step.max_context, "requests": step.n_requests, "rows": step.n_tokens}
+        meta = self._batch_facts(step)
         att = ops.attention_dv(y[:, :self.q_dim], k_cache, v_cache, g.block_table, step.row_req, step.positions, s.heads,
                                s.kv_heads, s.maps, s.dim, s.vdim, s.scale, softcap=s.softcap, window=s.window,
                                out_dtype=torch.float32, meta=meta, exact=exact)

@@ -160,7 +160,7 @@ def test_attention_kernel_on_crafted_keys(dtype, maps, softcap):
     from jllm_serve_amd.kernels import ops
     act = act_type(dtype)
     torch.manual_seed(11 + maps)
-    H, G, dk, dv, page, T = 4, 2, 24, 40, 16, 700
+    H, G, dk, dv, page, T = 4, 2, 32, 40, 16, 700  # sizes the matrix-core kernel takes, in bfloat16
     QS, KS = H * maps, G * maps
     n_pages = 64
     table = _pages(T, page, n_pages, 5)
@@ -192,10 +192,14 @@ def test_attention_kernel_on_crafted_keys(dtype, maps, softcap):
     bt = torch.tensor([table + [0] * 3], dtype=torch.int32, device=DEV)
     pos = torch.arange(T, dtype=torch.int32, device=DEV)
     req = torch.zeros(T, dtype=torch.int32, device=DEV)
+    tiles = [v for r0 in range(0, T, 128) for v in (0, r0, min(128, T - r0), r0)]
     for exact in ((True,) if dtype == "float32" else (True, False)):
+        ops.reset_stats()
         got = ops.attention_dv(q.reshape(T, -1).to(DEV), kc.to(DEV), vc.to(DEV), bt, req, pos, H, G, maps, dk, dv, scale,
                                softcap=softcap, out_dtype=torch.float32, exact=exact,
-                               meta={"max_context": T, "requests": 1, "rows": T}).cpu().view(T, QS, dv)
+                               meta={"max_context": T, "requests": 1, "rows": T, "n_tiles": len(tiles) // 4,
+                                     "tiles_dev": torch.tensor(tiles, dtype=torch.int32, device=DEV)}).cpu().view(T, QS, dv)
+        assert exact or ops.stats()["ran"].get("jllm_attention_dv_bf16") == 1, "the matrix-core kernel did not take the step"
         assert bool(torch.isfinite(got).all()), "a place that no position owns was read"
         tol = 2e-5 if dtype == "float32" else 2e-2
         assert float((got.double() - want).abs().max()) <= tol * float(want.abs().max())
@@ -211,7 +215,9 @@ def test_attention_kernel_on_crafted_keys(dtype, maps, softcap):
         one = ops.attention_dv(q.reshape(T, -1).to(DEV)[sel].contiguous(), kc.to(DEV), vc.to(DEV), bt.repeat(len(rows), 1),
                                torch.arange(len(rows), dtype=torch.int32, device=DEV), pos[sel].contiguous(), H, G, maps, dk, dv,
                                scale, softcap=softcap, out_dtype=torch.float32, exact=exact,
-                               meta={"max_context": T, "requests": len(rows), "rows": len(rows), "single_rows": True}).cpu()
+                               meta={"max_context": T, "requests": len(rows), "rows": len(rows), "n_tiles": len(rows),
+                                     "tiles_dev": torch.tensor([v for i in range(len(rows)) for v in (i, i, 1, -1)],
+                                                               dtype=torch.int32, device=DEV)}).cpu()
         assert float((one.view(len(rows), QS, dv).double() - want[rows]).abs().max()) <= tol * float(want.abs().max())
 
 
@@ -260,7 +266,7 @@ def test_qkv_prepare_options():
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("H, G, dk, dv", [(2, 1, 16, 8), (3, 3, 40, 24), (2, 2, 128, 128), (1, 1, 7, 5)])
+@pytest.mark.parametrize("H, G, dk, dv", [(2, 1, 16, 8), (3, 3, 40, 24), (2, 2, 128, 128), (1, 1, 7, 5), (2, 1, 200, 40)])
 def test_delta_rule_recalls_a_far_memory(dtype, H, G, dk, dv):
     """The kernel against the plain recurrence over 600 tokens cut into portions, with inputs chosen so that a fault
     shows: the first token writes a value along a key that no later token touches, nothing decays, and the last token
@@ -315,8 +321,9 @@ def test_delta_rule_recalls_a_far_memory(dtype, H, G, dk, dv):
             qkv = torch.cat([r[0][at:at + n] for r in reqs])
             proj = torch.cat([r[1][at:at + n] for r in reqs])
             row_req = torch.tensor([0] * n + [1] * n, dtype=torch.int32, device=DEV)
-            out = ops.gated_delta(dev(qkv), dev(proj), 0, H * dv, H * dv + H, dev(a_log), dev(dt_bias), dev(gain), state, row_req,
-                                  slots, 2, H, G, dk, dv, eps).cpu()
+            pd = dev(proj)
+            raw = ops.gated_delta(dev(qkv), pd, H * dv, H * dv + H, dev(a_log), dev(dt_bias), state, row_req, slots, 2, H, G, dk, dv)
+            out = ops.heads_finish(raw, H, 1, dv, act, normed=True, eps=eps, gain=dev(gain), gate=pd[:, :H * dv], gate_fn="silu").cpu()
             got[0].append(out[:n])
             got[1].append(out[n:])
             at += n

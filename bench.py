@@ -17,6 +17,8 @@ request sets served to the end, with the time the roofline allows for their pass
 `--no-serve`, `--no-fp32`, `--no-long` and `--no-shapes` leave groups out; `--temperature/--top-k/--top-p` make the
 main decode run a sampled one.
 
+`--workload compare --design kebepel [--size 2k|4k]` measures a Kebepel model (parallel attention / delta-rule layers and
+differential attention layers) beside the Qwen3 dense model of the same width, heads and feed-forward.
 `--workload compare [--size 2k|4k]` is another run altogether: a Miforax model (latent attention with a window, dense
 and table-routed expert layers in turn) beside the closest model the engine had before, a Qwen3 dense model with the
 same width, layers, heads, window and feed-forward width, both with random weights: prefill of 2,048 tokens and
@@ -166,6 +168,89 @@ class LatentWork:
         return 2.0 * rows * per_row + 2.0 * self.H * (self.hd + self.z["kv_rank"]) * self.L * pairs + 2.0 * self.V * self.d * selected
 
 
+KEBEPEL_SIZES = {  # layer sizes that resemble released models with a delta-rule mixer beside attention
+    "2k": dict(width=2048, layers=4, heads=16, kv_heads=8, dim=128, vdim=128, d_heads=8, d_kv_heads=4, d_vdim=256,
+               r_heads=16, r_kv_heads=8, conv=4, ff=8192, vocab=32768, window=0),
+    "4k": dict(width=4096, layers=4, heads=32, kv_heads=8, dim=128, vdim=128, d_heads=16, d_kv_heads=4, d_vdim=256,
+               r_heads=32, r_kv_heads=16, conv=4, ff=12288, vocab=32768, window=0),
+}
+
+
+def kebepel_config(z: dict) -> dict:
+    """Parallel layers (capped attention with rotation beside a gated delta rule) with a differential attention as
+    every second layer's mixer from the second on; every layer has a dense feed-forward."""
+    left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": z["dim"] ** -0.5,
+            "softcap": 50.0, "rot": {"base": 5e5, "dims": z["dim"], "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+    right = {"heads": z["r_heads"], "kv_heads": z["r_kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "conv": z["conv"]}
+    par = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.5}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+    att = {"type": "attention", "mixer": {"heads": z["d_heads"], "kv_heads": z["d_kv_heads"], "dim": z["dim"], "vdim": z["d_vdim"],
+                                          "scale": z["dim"] ** -0.5, "diff": 0.3, "q_temp": {"coef": 0.5, "every": 128}},
+           "mlp": {"kind": "dense", "ff": z["ff"]}}
+    return {"architecture": "Kebepel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "max_positions": 8192,
+            "layers": [att if i % 2 else par for i in range(z["layers"])]}
+
+
+class KebepelWork:
+    """Bytes and flops of passes over a Kebepel model of the sizes ``z`` (the interface of ``Work``). A decode step reads
+    every weight, per request the cached keys and values of every layer, and reads and writes the delta rule's matrices
+    (fp32); a row costs 2 flops per weight, per (row, key) pair 2 (dk + dv) per score map, and in the delta rule 6 dk
+    dv per head (two products with the matrix and its update)."""
+
+    def __init__(self, z: dict, dtype: str):
+        self.z = z
+        self.L, self.d, self.H, self.Hkv, self.F, self.V, self.hd = z["layers"], z["width"], z["heads"], z["kv_heads"], z["ff"], z["vocab"], z["dim"]
+        self.esize = 2 if dtype == "bf16" else 4
+        self.dtype = dtype
+        d, dk, dv = self.d, z["dim"], z["vdim"]
+        left = (z["heads"] * dk + z["kv_heads"] * (dk + dv) + z["heads"] * dv) * d + d * z["heads"] * dv
+        right = (2 * z["r_kv_heads"] * dk + 2 * z["r_heads"] * dv + 2 * z["r_heads"]) * d + d * z["r_heads"] * dv
+        diff = (2 * z["d_heads"] * dk + z["d_kv_heads"] * (2 * dk + z["d_vdim"]) + z["d_heads"] * z["d_vdim"]) * d + d * z["d_heads"] * z["d_vdim"]
+        self.n_att = self.L // 2
+        self.n_par = self.L - self.n_att
+        self.per_row = self.n_par * (left + right) + self.n_att * diff + self.L * 3 * d * z["ff"]
+        self.kv_bytes_per_token = (self.n_par * z["kv_heads"] * (dk + dv) + self.n_att * z["d_kv_heads"] * (2 * dk + z["d_vdim"])) * self.esize
+        self.state_bytes = self.n_par * z["r_heads"] * dk * dv * 4 * 2
+        self.pair_flops = self.n_par * 2 * z["heads"] * (dk + dv) + self.n_att * 2 * 2 * z["d_heads"] * (dk + z["d_vdim"])
+        self.row_flops = self.n_par * 6 * z["r_heads"] * dk * dv
+        self.weight_bytes = (self.per_row + self.V * d) * self.esize
+
+    def decode_bytes(self, tokens_held: float, batch: int = 0) -> float:
+        return self.weight_bytes + self.kv_bytes_per_token * tokens_held + self.state_bytes * max(batch, 1)
+
+    def pairs(self, T: int) -> float:
+        return T * (T + 1) / 2.0
+
+    def flops(self, rows: float, pairs: float, selected: float) -> float:
+        return rows * (2.0 * self.per_row + self.row_flops) + self.pair_flops * pairs + 2.0 * self.V * self.d * selected
+
+
+def compare_kebepel(args) -> dict:
+    """``--workload compare --design kebepel``: the Kebepel model of ``--size`` and the Qwen3 dense model of the same
+    width, heads, head size and feed-forward, one after the other: prefill of 2,048 tokens in one portion, decoding at
+    batch 8 and 64 behind prompts of 1,152 tokens."""
+    z = KEBEPEL_SIZES[args.size]
+    ctx = 4096
+    decodes = [dict(key=f"b{B}", batch=B, prompt_len=1152, steps=args.point_steps, warmup=4) for B in (8, 64)]
+    prefills = [dict(key="main", tokens=2048, portion=2048)]
+    out = {"metric": f"Kebepel beside Qwen3 dense at equal sizes ({args.size})", "unit": "tok/s", "n_gpus": 1, "dtype": "bf16",
+           "data": "synthetic (random weights N(0,0.02), uniform-random token ids)", "higher_is_better": True,
+           "config": {"size": args.size, **z, "context": ctx, "page_size": PAGE}, "models": {}}
+    qwen = qwen_like_config(z)
+    qwen.update(use_sliding_window=False)
+    for name, shape, work in (("kebepel", kebepel_config(z), KebepelWork(z, "bf16")), ("qwen3_dense", qwen, None)):
+        r = steady(args, name, "bf16", 0, ctx, decodes, prefills, shape=shape, work=work)
+        m = {"prefill_2048_tok_s": r["prefill"]["main"]["value"], "prefill_2048_ms": r["prefill"]["main"]["ms"],
+             "prefill_flop_frac": r["prefill"]["main"]["frac"]}
+        for B in (8, 64):
+            s_, held, by = r["decode"][f"b{B}"]
+            m[f"decode_b{B}_tok_s"] = round(B / s_, 1)
+            m[f"decode_b{B}_ms"] = round(s_ * 1e3, 3)
+            m[f"decode_b{B}_hbm_frac"] = round(by / s_ / HBM_PEAK, 4)
+        out["models"][name] = m
+    out["value"] = out["models"]["kebepel"]["decode_b8_tok_s"]
+    return out
+
+
 def compare_workload(args) -> dict:
     """``--workload compare``: the Miforax model of ``--size`` and the Qwen3 dense model of the same sizes, one after
     the other: prefill of 2,048 tokens in one portion, decoding at batch 8 and 64 with every window full."""
@@ -313,6 +398,8 @@ def main() -> int:
                     help="steady: timed decode steps at a fixed batch (the default run); serve: a request set run to the end; "
                          "compare: a Miforax model beside the Qwen3 dense model of the same sizes")
     ap.add_argument("--size", default="2k", choices=sorted(COMPARE_SIZES), help="compare: which sizes")
+    ap.add_argument("--design", default="miforax", choices=["miforax", "kebepel"],
+                    help="compare: which design stands beside the Qwen3 dense model of the same sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -322,7 +409,7 @@ def main() -> int:
         print(json.dumps(serve_workload(args)))
         return 0
     if args.workload == "compare":
-        print(json.dumps(compare_workload(args)))
+        print(json.dumps(compare_kebepel(args) if args.design == "kebepel" else compare_workload(args)))
         return 0
 
     import torch

@@ -6,23 +6,27 @@
 //   short_conv_silu      y[t, c] = silu(sum_j taps[c, K - 1 - j] x[t - j, c]); inputs before the step's first row of a
 //                        request come from that request's state, inputs before position 0 are the state's zeros
 //   short_conv_advance   the state's K - 1 inputs per channel move on by the request's rows of this step
+//   delta_prepare        per (row, key head), what the recurrence would otherwise compute in every lane of every wave:
+//                          q <- q / sqrt(sum q^2 + 1e-6) / sqrt(dk), k <- k / sqrt(sum k^2 + 1e-6), q . k, and per head
+//                          beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias)); all in fp32
 //   gated_delta          token by token, with S [dk, dv] in registers:
-//                          q <- q / sqrt(sum q^2 + 1e-6) / sqrt(dk), k <- k / sqrt(sum k^2 + 1e-6)
-//                          beta = sigmoid(b), g = exp(-exp(A_log) * softplus(a + dt_bias))
 //                          S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q
 //                        computed as  S^T k and S^T q of the old S in one pass, o = g S^T q + (k . q) u.
-//                        The columns of S never meet: column j only needs v[j], so a workgroup is ONE wave that owns 16
-//                        value columns of one head of one request (4 lanes per column, a quarter of the key rows
-//                        each) and walks the request's rows without a barrier; a step of one request and 16 heads of
-//                        128 x 128 is 128 such waves. The read-out o goes out raw in fp32; the heads' norm, gain and
-//                        gate need all columns of a head and are the finishing kernel's (attention_dv.hip).
+//                        The columns of S never meet: column j only needs v[j]. A workgroup of four waves owns 16 value
+//                        columns of one head of one request: a wave 4 of them, 16 lanes per column with a sixteenth of
+//                        the key rows each (sums over a column's lanes are moves inside a row of 16 lanes). It walks
+//                        the request's rows in chunks of 16 that are requested a chunk ahead and shared through LDS.
+//                        One request and 16 heads of 128 x 128 are 512 waves. The read-out o goes out raw in fp32; the
+//                        heads' norm, gain and gate need all columns of a head and are the finishing kernel's
+//                        (attention_dv.hip).
 #include <math.h>
 
 #include "common.h"
 
 #define CONV_MAX_TAPS 16
-#define GDR_COLS 16   // value columns of a wave
-#define GDR_PARTS 4   // lanes per column: each owns a quarter of the key rows
+#define GDR_COLS 16    // value columns of a workgroup (4 per wave)
+#define GDR_PARTS 16   // lanes per column: each owns a sixteenth of the key rows
+#define GDR_CHUNK 16   // rows staged at a time
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
@@ -114,128 +118,187 @@ extern "C" int jllm_short_conv(const void* x, int ldx, void* y, int ldy, int dty
 
 // ---------------------------------------------------------------------------------------------------------------------
 
+// prep row: qn (kv_heads x dk) | kn (kv_heads x dk) | g (heads) | beta (heads) | q . k (kv_heads)
+template <typename T, typename TW>
+__global__ __launch_bounds__(64) void delta_prepare_kernel(const T* __restrict__ conv, int ldc, const T* __restrict__ proj,
+                                                           int ldp, int a_off, int b_off, const TW* __restrict__ a_log,
+                                                           const TW* __restrict__ dt_bias, float* __restrict__ prep, int ldq,
+                                                           int heads, int kv_heads, int dk) {
+  const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+  const T* q = conv + (size_t)row * ldc + (size_t)g * dk;
+  const T* k = conv + (size_t)row * ldc + (size_t)(kv_heads + g) * dk;
+  float sq = 0.f, sk = 0.f, qk = 0.f;
+  for (int i = lane; i < dk; i += 64) {
+    const float a = ldf(q, i), b = ldf(k, i);
+    sq = fmaf(a, a, sq);
+    sk = fmaf(b, b, sk);
+    qk = fmaf(a, b, qk);
+  }
+  sq = wave_sum(sq), sk = wave_sum(sk), qk = wave_sum(qk);
+  const float rq = (1.0f / sqrtf((float)dk)) / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
+  float* out = prep + (size_t)row * ldq;
+  for (int i = lane; i < dk; i += 64) {
+    out[(size_t)g * dk + i] = ldf(q, i) * rq;
+    out[(size_t)(kv_heads + g) * dk + i] = ldf(k, i) * rk;
+  }
+  const int per = heads / kv_heads;
+  float* tail = out + (size_t)2 * kv_heads * dk;
+  for (int j = lane; j < per; j += 64) {
+    const int h = g * per + j;
+    const float z = ldf(proj + (size_t)row * ldp, a_off + h) + ldf(dt_bias, h);
+    const float sp = z > 20.f ? z : log1pf(expf(z));
+    tail[h] = expf(-expf(ldf(a_log, h)) * sp);
+    tail[heads + h] = 1.0f / (1.0f + expf(-ldf(proj + (size_t)row * ldp, b_off + h)));
+  }
+  if (lane == 0) tail[2 * heads + g] = qk * rq * rk;
+}
+
 struct GdrArgs {
-  const void* qkv;   // [rows, ldc]: q (kv_heads x dk) | k (kv_heads x dk) | v (heads x dv), convolved
+  const void* conv;   // [rows, ldc]: q | k | v (heads x dv) convolved; only v is read here
   int ldc;
-  const void* proj;  // [rows, ldp]: the projection's row, which holds a and b (heads each) at their offsets
-  int ldp, a_off, b_off;
-  const void* a_log;    // [heads]
-  const void* dt_bias;  // [heads]
-  float* state;         // [slots, heads, dk, dv]
-  float* out;           // [rows, ldo]: heads x dv, the raw read-out
+  const float* prep;  // [rows, ldq]: what delta_prepare left
+  int ldq;
+  float* state;       // [slots, heads, dk, dv]
+  float* out;         // [rows, ldo]: heads x dv, the raw read-out
   int ldo;
   const int* row_req;
   const int* state_slots;
   int n_rows, heads, kv_heads, dk, dv;
 };
 
-// what a lane needs of one row: its quarter of q and k, its column's v, the head's a and b
-template <typename T, int E>
-struct GdrRow {
-  float q[E], k[E], v, a, b;
-  __device__ __forceinline__ void load(const GdrArgs& A, size_t row, int kvh, int h, int i0, int col, bool col_on) {
-    const T* cr = (const T*)A.qkv + row * A.ldc;
-    const T* qr = cr + (size_t)kvh * A.dk;
-    const T* kr = cr + (size_t)(A.kv_heads + kvh) * A.dk;
-#pragma unroll
-    for (int e = 0; e < E; ++e) {
-      const bool on = i0 + e < A.dk;
-      q[e] = on ? ldf(qr, i0 + e) : 0.f;
-      k[e] = on ? ldf(kr, i0 + e) : 0.f;
-    }
-    v = col_on ? ldf(cr, (size_t)2 * A.kv_heads * A.dk + (size_t)h * A.dv + col) : 0.f;
-    const T* pr = (const T*)A.proj + row * A.ldp;
-    a = ldf(pr, A.a_off + h);
-    b = ldf(pr, A.b_off + h);
-  }
-};
-
-__device__ __forceinline__ float parts_sum(float v) {  // over the four lanes of a column, the same in all of them
-  v += __shfl_xor(v, 16, 64);
-  v += __shfl_xor(v, 32, 64);
-  return v;
+__device__ __forceinline__ float row16_sum(float d) {  // over a row of 16 lanes, left in all of them
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0xB1, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x4E, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x141, 0xF, 0xF, true));
+  d += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, d), 0x140, 0xF, 0xF, true));
+  return d;
 }
 
-// lane = part * 16 + c: column blockIdx.z * 16 + c, key rows part * E .. + E
-template <typename T, typename TW, int E, bool AHEAD>
-__global__ __launch_bounds__(64) void gated_delta_kernel(GdrArgs A) {
-  const int lane = threadIdx.x;
-  const int c = lane & (GDR_COLS - 1), part = lane / GDR_COLS;
+// thread = wave * 64 + c * 16 + part: column blockIdx.z * 16 + wave * 4 + c, key rows part * E .. + E
+template <typename T, int E>
+__global__ __launch_bounds__(256) void gated_delta_kernel(GdrArgs A) {
+  constexpr int C = GDR_CHUNK;
+  constexpr int DKP = GDR_PARTS * E;              // the key size, padded with zeros
+  constexpr int ROWF = 2 * DKP + GDR_COLS + 4;    // q | k | v of the workgroup's columns | g | beta | q . k | -
+  constexpr int NQK = C * 2 * DKP / 256;
+  __shared__ __align__(16) float sm[C * ROWF];
+  const int tid = threadIdx.x;
+  const int part = tid & 15, cw = tid >> 4;  // cw: the column within the workgroup
   const int req = blockIdx.x, h = blockIdx.y;
-  const int col = blockIdx.z * GDR_COLS + c;
+  const int col0 = blockIdx.z * GDR_COLS;
+  const int col = col0 + cw;
   const bool col_on = col < A.dv;
   int lo, n;
   rows_of_request(A.row_req, A.n_rows, req, lo, n);
   if (n == 0) return;
+  const int dk = A.dk;
   const int kvh = h / (A.heads / A.kv_heads);
   const int i0 = part * E;
-  float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * A.dk * A.dv;
+  float* S_at = A.state + ((size_t)A.state_slots[req] * A.heads + h) * dk * A.dv;
   float S[E];
 #pragma unroll
-  for (int e = 0; e < E; ++e) S[e] = (col_on && i0 + e < A.dk) ? S_at[(size_t)(i0 + e) * A.dv + col] : 0.f;
-  const float decay_rate = expf(ldf((const TW*)A.a_log, h));
-  const float dtb = ldf((const TW*)A.dt_bias, h);
-  const float q_scale = 1.0f / sqrtf((float)A.dk);
-  GdrRow<T, E> cur, nxt;
-  cur.load(A, (size_t)lo, kvh, h, i0, col, col_on);
-  for (int r = 0; r < n; ++r) {
-    if (AHEAD && r + 1 < n) nxt.load(A, (size_t)(lo + r + 1), kvh, h, i0, col, col_on);  // in flight under this row's sums
-    float sq = 0.f, sk = 0.f, qk = 0.f, dk_ = 0.f, dq_ = 0.f;
+  for (int e = 0; e < E; ++e) S[e] = (col_on && i0 + e < dk) ? S_at[(size_t)(i0 + e) * A.dv + col] : 0.f;
+  const T* conv = (const T*)A.conv;
+  const size_t q_at = (size_t)kvh * dk, k_at = (size_t)(A.kv_heads + kvh) * dk;
+  const size_t tail_at = (size_t)2 * A.kv_heads * dk;
+  const size_t v_at = (size_t)2 * A.kv_heads * dk + (size_t)h * A.dv + col0;
+  float rqk[NQK], rv, rs;
+  auto request = [&](int r0) {  // rows r0 .. r0 + C of the request, as far as it has them
+    const int have = min(C, n - r0);
 #pragma unroll
-    for (int e = 0; e < E; ++e) {
-      sq = fmaf(cur.q[e], cur.q[e], sq);
-      sk = fmaf(cur.k[e], cur.k[e], sk);
-      qk = fmaf(cur.q[e], cur.k[e], qk);
-      dk_ = fmaf(S[e], cur.k[e], dk_);
-      dq_ = fmaf(S[e], cur.q[e], dq_);
+    for (int j = 0; j < NQK; ++j) {
+      const int idx = tid + 256 * j;
+      const int t = idx / (2 * DKP), w = idx % (2 * DKP);
+      const int i = w % DKP;
+      rqk[j] = (t < have && i < dk) ? A.prep[(size_t)(lo + r0 + t) * A.ldq + (w < DKP ? q_at : k_at) + i] : 0.f;
     }
-    sq = parts_sum(sq), sk = parts_sum(sk), qk = parts_sum(qk), dk_ = parts_sum(dk_), dq_ = parts_sum(dq_);
-    const float rq = q_scale / sqrtf(sq + 1e-6f), rk = 1.0f / sqrtf(sk + 1e-6f);
-    const float z = cur.a + dtb;
-    const float sp = z > 20.f ? z : log1pf(expf(z));
-    const float g = expf(-decay_rate * sp);
-    const float beta = 1.0f / (1.0f + expf(-cur.b));
-    const float u = beta * (cur.v - g * (dk_ * rk));
-    const float o = fmaf(g, dq_ * rq, qk * rq * rk * u);
-    const float ku = u * rk;
+    {
+      const int t = tid / GDR_COLS, cc = tid % GDR_COLS;
+      rv = (t < have && col0 + cc < A.dv) ? ldf(conv + (size_t)(lo + r0 + t) * A.ldc + v_at, cc) : 0.f;
+    }
+    rs = 0.f;
+    if (tid < 3 * C && tid / 3 < have) {
+      const int which = tid % 3;  // g, beta, q . k
+      rs = A.prep[(size_t)(lo + r0 + tid / 3) * A.ldq + tail_at + (which == 0 ? h : which == 1 ? A.heads + h : 2 * A.heads + kvh)];
+    }
+  };
+  auto stage = [&]() {
 #pragma unroll
-    for (int e = 0; e < E; ++e) S[e] = fmaf(cur.k[e], ku, g * S[e]);
-    if (part == 0 && col_on) A.out[(size_t)(lo + r) * A.ldo + (size_t)h * A.dv + col] = o;
-    if (AHEAD)
-      cur = nxt;
-    else if (r + 1 < n)
-      cur.load(A, (size_t)(lo + r + 1), kvh, h, i0, col, col_on);
+    for (int j = 0; j < NQK; ++j) {
+      const int idx = tid + 256 * j;
+      sm[(idx / (2 * DKP)) * ROWF + idx % (2 * DKP)] = rqk[j];
+    }
+    sm[(tid / GDR_COLS) * ROWF + 2 * DKP + tid % GDR_COLS] = rv;
+    if (tid < 3 * C) sm[(tid / 3) * ROWF + 2 * DKP + GDR_COLS + tid % 3] = rs;
+  };
+  request(0);
+  for (int r0 = 0; r0 < n; r0 += C) {
+    __syncthreads();  // the chunk before has been read
+    stage();
+    __syncthreads();
+    if (r0 + C < n) request(r0 + C);  // in flight while this chunk is worked through
+    const int have = min(C, n - r0);
+    for (int t = 0; t < have; ++t) {
+      const float* row = sm + t * ROWF;
+      float q[E], k[E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        q[e] = row[i0 + e];
+        k[e] = row[DKP + i0 + e];
+      }
+      const float v = row[2 * DKP + cw], g = row[2 * DKP + GDR_COLS], beta = row[2 * DKP + GDR_COLS + 1];
+      const float qk = row[2 * DKP + GDR_COLS + 2];
+      float sk_ = 0.f, sq_ = 0.f;
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        sk_ = fmaf(S[e], k[e], sk_);
+        sq_ = fmaf(S[e], q[e], sq_);
+      }
+      sk_ = row16_sum(sk_), sq_ = row16_sum(sq_);
+      const float u = beta * (v - g * sk_);
+      const float o = fmaf(g, sq_, qk * u);
+#pragma unroll
+      for (int e = 0; e < E; ++e) S[e] = fmaf(k[e], u, g * S[e]);
+      if (part == 0 && col_on) A.out[(size_t)(lo + r0 + t) * A.ldo + (size_t)h * A.dv + col] = o;
+    }
   }
 #pragma unroll
   for (int e = 0; e < E; ++e)
-    if (col_on && i0 + e < A.dk) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
+    if (col_on && i0 + e < dk) S_at[(size_t)(i0 + e) * A.dv + col] = S[e];
 }
 
+// prep: fp32 scratch [rows, >= 2 kv_heads dk + 2 heads + kv_heads]
 extern "C" int jllm_gated_delta(const void* qkv, int ldc, const void* proj, int ldp, int a_off, int b_off, int dtype,
-                                const void* a_log, const void* dt_bias, int w_dtype, float* state, float* out, int ldo,
-                                const int* row_req, const int* state_slots, int n_rows, int n_requests, int heads,
-                                int kv_heads, int dk, int dv, hipStream_t stream) {
+                                const void* a_log, const void* dt_bias, int w_dtype, float* prep, int ldq, float* state,
+                                float* out, int ldo, const int* row_req, const int* state_slots, int n_rows, int n_requests,
+                                int heads, int kv_heads, int dk, int dv, hipStream_t stream) {
   if (n_rows <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads || heads > 65535) JLLM_FAIL("gated_delta: %d heads over %d key heads", heads, kv_heads);
-  if (dk <= 0 || dk > GDR_PARTS * 64 || dv <= 0 || dv > GDR_COLS * 65535) JLLM_FAIL("gated_delta: key size %d (1..%d are taken), value size %d", dk, GDR_PARTS * 64, dv);
+  if (dk <= 0 || dk > GDR_PARTS * 16 || dv <= 0 || dv > GDR_COLS * 65535) JLLM_FAIL("gated_delta: key size %d (1..%d are taken), value size %d", dk, GDR_PARTS * 16, dv);
   if (n_requests <= 0 || n_requests > n_rows) JLLM_FAIL("gated_delta: %d requests in %d rows", n_requests, n_rows);
-  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || ldp < a_off + heads || ldp < b_off + heads || a_off < 0 || b_off < 0)
+  if (ldc < 2 * kv_heads * dk + heads * dv || ldo < heads * dv || ldp < a_off + heads || ldp < b_off + heads || a_off < 0 || b_off < 0 ||
+      ldq < 2 * kv_heads * dk + 2 * heads + kv_heads)
     JLLM_FAIL("gated_delta: short rows");
-  GdrArgs A{qkv, ldc, proj, ldp, a_off, b_off, a_log, dt_bias, state, out, ldo, row_req, state_slots, n_rows, heads, kv_heads, dk, dv};
-  dim3 grid(n_requests, heads, (dv + GDR_COLS - 1) / GDR_COLS);
-  const int per_lane = (dk + GDR_PARTS - 1) / GDR_PARTS;
-#define GDR_LAUNCH(E, AHEAD) gated_delta_kernel<T, TW, E, AHEAD><<<grid, 64, 0, stream>>>(A)
   JLLM_DISPATCH_1(dtype, T, {
     JLLM_DISPATCH_1(w_dtype, TW, {
-      if (per_lane <= 8)
-        GDR_LAUNCH(8, true);
-      else if (per_lane <= 16)
-        GDR_LAUNCH(16, true);
-      else if (per_lane <= 32)
-        GDR_LAUNCH(32, true);
-      else
-        GDR_LAUNCH(64, false);
+      delta_prepare_kernel<T, TW><<<dim3(n_rows, kv_heads), 64, 0, stream>>>((const T*)qkv, ldc, (const T*)proj, ldp, a_off, b_off,
+                                                                            (const TW*)a_log, (const TW*)dt_bias, prep, ldq, heads,
+                                                                            kv_heads, dk);
     })
+  })
+  GdrArgs A{qkv, ldc, prep, ldq, state, out, ldo, row_req, state_slots, n_rows, heads, kv_heads, dk, dv};
+  dim3 grid(n_requests, heads, (dv + GDR_COLS - 1) / GDR_COLS);
+  const int per_lane = (dk + GDR_PARTS - 1) / GDR_PARTS;
+#define GDR_LAUNCH(E) gated_delta_kernel<T, E><<<grid, 256, 0, stream>>>(A)
+  JLLM_DISPATCH_1(dtype, T, {
+    if (per_lane <= 2)
+      GDR_LAUNCH(2);
+    else if (per_lane <= 4)
+      GDR_LAUNCH(4);
+    else if (per_lane <= 8)
+      GDR_LAUNCH(8);
+    else
+      GDR_LAUNCH(16);
   })
 #undef GDR_LAUNCH
   JLLM_CHECK_LAUNCH("gated_delta");

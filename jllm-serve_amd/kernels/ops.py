@@ -80,7 +80,7 @@ def _declare(lib) -> None:
         "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
         "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _P, _I, _I, _P],
         "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
-        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
+        "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -1199,8 +1199,8 @@ MAX_CONV_TAPS = 16
 
 
 def check_gated_delta_shape(heads: int, kv_heads: int, dk: int, dv: int, taps: int) -> None:
-    """Raises when the delta-rule kernels do not take these sizes (asked when a model is built): a wave keeps a
-    quarter of the key rows of 16 value columns per lane."""
+    """Raises when the delta-rule kernels do not take these sizes (asked when a model is built): a lane keeps a
+    sixteenth of the key rows of one value column."""
     if heads <= 0 or kv_heads <= 0 or heads % kv_heads != 0:
         raise KernelError(f"gated delta rule: {heads} heads over {kv_heads} key heads")
     if not 1 <= taps <= MAX_CONV_TAPS:
@@ -1263,9 +1263,11 @@ def gated_delta(qkv: torch.Tensor, proj: torch.Tensor, a_off: int, b_off: int, a
     out = torch.empty((T, heads * dv), dtype=torch.float32, device=qkv.device)
     if T == 0:
         return out
+    # what the preparing kernel leaves for the recurrence: unit q and k, decay, write strength and q . k, in fp32
+    prep = torch.empty((T, 2 * kv_heads * dk + 2 * heads + kv_heads), dtype=torch.float32, device=qkv.device)
     _call("jllm_gated_delta", _ptr(qkv), qkv.stride(0), _ptr(proj), proj.stride(0), int(a_off), int(b_off), _code(qkv.dtype),
-          _ptr(a_log), _ptr(dt_bias), wd, _ptr(state), _ptr(out), out.stride(0), _ptr(row_req), _ptr(state_slots), T,
-          int(n_requests), heads, kv_heads, dk, dv, _stream())
+          _ptr(a_log), _ptr(dt_bias), wd, _ptr(prep), prep.stride(0), _ptr(state), _ptr(out), out.stride(0), _ptr(row_req),
+          _ptr(state_slots), T, int(n_requests), heads, kv_heads, dk, dv, _stream())
     return out
 
 

@@ -14,8 +14,8 @@
 //                    to absolute positions, wave w takes the blocks with c % 4 == w, the four waves' results are merged
 //                    in wave order: a row's result depends only on its own position and keys
 //   heads_finish     per (row, head): with two maps o = a1 - lambda * a2; optionally o / sqrt(mean(o^2) + eps) * gain;
-//                    optionally times sigmoid(gate) or silu(gate); written as the output product's input (other mixers
-//                    whose heads end this way use it too)
+//                    optionally times sigmoid(gate) or silu(gate), times a constant; written as the output product's
+//                    input (other mixers whose heads end this way use it too)
 //
 // Cache layout of one layer run: keys [page][key slot][page_size][dk], values [page][value head][page_size][dv];
 // position j of request r lives in page block_table[r][j / page_size] at offset j % page_size.
@@ -232,7 +232,7 @@ template <typename TA, typename TG, typename TW, typename TO>
 __global__ __launch_bounds__(64) void heads_finish_kernel(const TA* __restrict__ att, int lda, int maps, int dv,
                                                           float lambda, int normed, float eps, float norm_mul,
                                                           const TW* __restrict__ gain, const TG* __restrict__ gate, int ldg,
-                                                          int gate_fn, TO* __restrict__ out, int ldo) {
+                                                          int gate_fn, float out_mul, TO* __restrict__ out, int ldo) {
   const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
   const TA* a = att + (size_t)t * lda + (size_t)h * maps * dv;
   float ss = 0.f;
@@ -254,14 +254,14 @@ __global__ __launch_bounds__(64) void heads_finish_kernel(const TA* __restrict__
       const float z = ldf(gate + (size_t)t * ldg, (size_t)h * dv + j);
       o *= (gate_fn == 1 ? z : 1.0f) / (1.0f + expf(-z));  // 0: sigmoid(z), 1: silu(z)
     }
-    stf(out + (size_t)t * ldo, (size_t)h * dv + j, o);
+    stf(out + (size_t)t * ldo, (size_t)h * dv + j, o * out_mul);
   }
 }
 
 // att [rows, lda]: heads x maps x dv per row; gate [rows, ldg]: heads x dv per row or null; out [rows, ldo]
 extern "C" int jllm_heads_finish(const void* att, int lda, int att_dtype, int n_tokens, int heads, int maps, int dv,
                                  float lambda, int normed, float eps, float norm_mul, const void* gain, int gain_dtype,
-                                 const void* gate, int ldg, int gate_dtype, int gate_fn, void* out, int ldo, int out_dtype,
+                                 const void* gate, int ldg, int gate_dtype, int gate_fn, float out_mul, void* out, int ldo, int out_dtype,
                                  hipStream_t stream) {
   if (n_tokens <= 0) return 0;
   if (heads <= 0 || heads > 65535 || dv <= 0 || (maps != 1 && maps != 2)) JLLM_FAIL("heads_finish: %d heads of %d with %d maps (one or two are taken)", heads, dv, maps);
@@ -273,7 +273,7 @@ extern "C" int jllm_heads_finish(const void* att, int lda, int att_dtype, int n_
       JLLM_DISPATCH_1(gain_dtype, TW, {
         JLLM_DISPATCH_1(out_dtype, TO, {
           heads_finish_kernel<TA, TG, TW, TO><<<grid, 64, 0, stream>>>((const TA*)att, lda, maps, dv, lambda, normed, eps, norm_mul,
-                                                                      (const TW*)gain, (const TG*)gate, ldg, gate_fn, (TO*)out, ldo);
+                                                                      (const TW*)gain, (const TG*)gate, ldg, gate_fn, out_mul, (TO*)out, ldo);
         })
       })
     })

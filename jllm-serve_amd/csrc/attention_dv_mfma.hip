@@ -15,6 +15,12 @@
 // The probabilities, rounded to bf16, are already laid out as the B operand of O^T[dim][row] += V^T P^T, whose A
 // operand is read from V with the transposing LDS load (ds_read_b64_tr_b16). dk and dv are independent: dk in steps
 // of 16 (the K loop), dv in blocks of 32 (the accumulators), both up to 256.
+//
+// Steps of single rows have few tiles with long chains of blocks: there gridDim.z workgroups share a tile's blocks
+// (`per_split` blocks each, in order), each leaves its unnormalised sums, maximum and sum in a scratch array, and a
+// second kernel merges them in the order of the splits. In such steps (`share` > 0) a workgroup also takes all query
+// heads that read the same key slot and value head at once, one per lane of its first wave, in the place of the rows
+// of a tile: the grid's x is then the key slot, and keys and values are read once for the whole group.
 #include <math.h>
 
 #include "common.h"
@@ -27,7 +33,7 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     const bf16_t* __restrict__ q, int ldq, float* __restrict__ out, int ldo, const bf16_t* __restrict__ kc,
     const bf16_t* __restrict__ vc, const int* __restrict__ block_table, int max_blocks, const int* __restrict__ tiles,
     const int* __restrict__ positions, int maps, int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window,
-    float scale, float softcap) {
+    float scale, float softcap, float* __restrict__ partial, int per_split, int share, int q_slots) {
   constexpr int DK = DK16 * 16;
   constexpr int DVP = DB * 32;
   constexpr int KLD = DK + 8;
@@ -43,13 +49,16 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
   const int* tile = tiles + (size_t)blockIdx.y * 4;
   const int req = tile[0], row0 = tile[1], nrows = tile[2];
   const int pos0 = tile[3] >= 0 ? tile[3] : positions[row0];
-  const int s = blockIdx.x;
-  const int vh = s / per_kv;
-  const int ks_ = vh * maps + s % maps;
   const int tid = threadIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
   const int qi = lane & 31, half = lane >> 5;
-  const int wq = wave * 32 + qi;
+  // share == 0: blockIdx.x is a query slot and the lanes of a wave are rows of the tile. share > 0 (tiles of one row):
+  // blockIdx.x is a key slot and lane qi < share of the first wave is the qi-th query head that reads it
+  const int vh = share ? (int)blockIdx.x / maps : (int)blockIdx.x / per_kv;
+  const int ks_ = share ? (int)blockIdx.x : vh * maps + (int)blockIdx.x % maps;
+  const int s = share ? (vh * share + min(qi, share - 1)) * maps + (int)blockIdx.x % maps : (int)blockIdx.x;
+  const int wq = share ? 0 : wave * 32 + qi;                    // the lane's row within the tile
+  const bool lane_on = share ? (wave == 0 && qi < share) : (wq < nrows);
   const int pos_q = pos0 + min(wq, nrows - 1);
   const int first_q = window > 0 ? max(0, pos_q + 1 - window) : 0;
   const int* tbl = block_table + (size_t)req * max_blocks;
@@ -58,15 +67,28 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
   const int wave_lo_pos = pos0 + min(nrows - 1, wave * 32);
   const int wave_hi = pos0 + min(nrows - 1, wave * 32 + 31);
   const int wave_first = window > 0 ? max(0, wave_hi + 1 - window) : 0;
-  const bool wave_on = wave * 32 < nrows;
+  const bool wave_on = share ? wave == 0 : wave * 32 < nrows;
   u32x4 qf[DK16];
   {
     const bf16_t* qr = q + (size_t)(row0 + min(wq, nrows - 1)) * ldq + (size_t)s * DK + half * 8;
 #pragma unroll
     for (int i = 0; i < DK16; ++i) qf[i] = *(const u32x4*)(qr + i * 16);
   }
-  const int kt_first = (k_lo / AT_KEYS) * AT_KEYS;
-  const int n_blocks = (k_hi - kt_first) / AT_KEYS + 1;
+  int kt_first = (k_lo / AT_KEYS) * AT_KEYS;
+  int n_blocks = (k_hi - kt_first) / AT_KEYS + 1;
+  if (partial) {  // this workgroup's share of the tile's blocks
+    const int b0 = blockIdx.z * per_split;
+    kt_first += b0 * AT_KEYS;
+    n_blocks = min(per_split, n_blocks - b0);
+    if (n_blocks <= 0) {  // nothing left for this split: it says so (the same for all threads: no barrier was met)
+      if (lane_on && half == 0) {
+        float* pr = partial + (((size_t)(row0 + wq) * q_slots + s) * gridDim.z + blockIdx.z) * (dv + 2);
+        pr[dv] = -INFINITY;
+        pr[dv + 1] = 0.f;
+      }
+      return;
+    }
+  }
   u32x4 kreg[KCH], vreg[VCH];
   int kpg[KCH], vpg[VCH];
   const int pmask = (1 << page_shift) - 1;
@@ -228,7 +250,22 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     if (more) store_block(buf ^ 1);
     __syncthreads();
   }
-  if (!wave_on || wq >= nrows) return;
+  if (!wave_on || !lane_on) return;
+  if (partial) {
+    float* pr = partial + (((size_t)(row0 + wq) * q_slots + s) * gridDim.z + blockIdx.z) * (dv + 2);
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) {
+        const int d = db * 32 + 8 * (e >> 2) + half * 4 + (e & 3);
+        if (d < dv) pr[d] = o[db][e];
+      }
+    if (half == 0) {
+      pr[dv] = m;
+      pr[dv + 1] = l;
+    }
+    return;
+  }
   const float inv = 1.0f / l;
   float* orow = out + (size_t)(row0 + wq) * ldo + (size_t)s * dv;
 #pragma unroll
@@ -240,10 +277,34 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     }
 }
 
+// partial [rows][q_slots][splits][dv + 2]: unnormalised sums, then the maximum (as an exponent of two) and the sum
+__global__ __launch_bounds__(64) void attention_dv_merge_kernel(const float* __restrict__ partial, int splits, int dv,
+                                                                float* __restrict__ out, int ldo) {
+  const int t = blockIdx.x, s = blockIdx.y, lane = threadIdx.x;
+  const float* pr = partial + ((size_t)t * gridDim.y + s) * splits * (dv + 2);
+  float mx = -INFINITY;
+  for (int z = 0; z < splits; ++z) mx = fmaxf(mx, pr[(size_t)z * (dv + 2) + dv]);
+  float l = 0.f;
+  for (int z = 0; z < splits; ++z) {
+    const float mz = pr[(size_t)z * (dv + 2) + dv];
+    if (mz != -INFINITY) l += pr[(size_t)z * (dv + 2) + dv + 1] * __builtin_amdgcn_exp2f(mz - mx);
+  }
+  const float inv = 1.0f / l;
+  for (int d = lane; d < dv; d += 64) {
+    float acc = 0.f;
+    for (int z = 0; z < splits; ++z) {
+      const float mz = pr[(size_t)z * (dv + 2) + dv];
+      if (mz != -INFINITY) acc = fmaf(pr[(size_t)z * (dv + 2) + d], __builtin_amdgcn_exp2f(mz - mx), acc);
+    }
+    out[(size_t)t * ldo + (size_t)s * dv + d] = acc * inv;
+  }
+}
+
 template <int DK16, int DB>
 static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq, float* out, int ldo, const bf16_t* kc,
                         const bf16_t* vc, const int* block_table, int max_blocks, const int* tiles, const int* positions, int maps,
-                        int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window, float scale, float softcap) {
+                        int per_kv, int k_slots, int v_heads, int dv, int page_shift, int window, float scale, float softcap,
+                        float* partial, int per_split, int share, int q_slots) {
   const size_t smem = (size_t)2 * AT_KEYS * ((DK16 * 16 + 8) + (DB * 32 + 32)) * sizeof(bf16_t);
   static bool raised = false;
   if (smem > 64 * 1024 && !raised) {
@@ -252,15 +313,19 @@ static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq,
     raised = true;
   }
   attention_dv_tiles_kernel<DK16, DB><<<grid, 256, smem, stream>>>(q, ldq, out, ldo, kc, vc, block_table, max_blocks, tiles, positions,
-                                                                 maps, per_kv, k_slots, v_heads, dv, page_shift, window, scale, softcap);
+                                                                 maps, per_kv, k_slots, v_heads, dv, page_shift, window, scale, softcap,
+                                                                 partial, per_split, share, q_slots);
   return 0;
 }
 
 // Returns 1 (declined) for sizes it does not take: dk a multiple of 16 up to 256, dv a multiple of 8 up to 256, bf16.
+// `splits` > 1 (tiles of single rows only): the workgroups of a tile take `per_split` key blocks each and `partial`
+// (fp32, rows x slots x splits x (dv + 2)) carries their results to the merge.
 extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ldo, const void* kcache, const void* vcache,
                                       const int* block_table, int max_blocks, const int* tiles, int n_tiles,
                                       const int* positions, int heads, int kv_heads, int maps, int dk, int dv, int page_size,
-                                      int window, float scale, float softcap, hipStream_t stream) {
+                                      int window, float scale, float softcap, int splits, int per_split, float* partial,
+                                      int n_rows, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || maps <= 0) JLLM_FAIL("attention: %d query heads over %d kv heads with %d maps", heads, kv_heads, maps);
   if ((dk & 15) || dk < 16 || dk > 256 || (dv & 7) || dv < 8 || dv > 256) return 1;
@@ -270,11 +335,16 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const int q_slots = heads * maps, per_kv = maps * (heads / kv_heads);
-  dim3 grid(q_slots, n_tiles);
+  if (splits > 1 && (!partial || per_split <= 0 || n_rows != n_tiles || splits > 65535)) JLLM_FAIL("attention: %d splits of %d blocks over %d tiles of %d rows", splits, per_split, n_tiles, n_rows);
+  if (splits <= 1) partial = nullptr;
+  // tiles of one row: the heads of a key slot share a workgroup (up to the 32 lanes that hold a tile's rows)
+  const int share = (n_rows == n_tiles && heads / kv_heads > 1 && heads / kv_heads <= 32) ? heads / kv_heads : 0;
+  dim3 grid(share ? kv_heads * maps : q_slots, n_tiles, partial ? splits : 1);
   const int db = (dv + 31) / 32;
   int rc = 1;
 #define AT_ARGS grid, stream, (const bf16_t*)q, ldq, out, ldo, (const bf16_t*)kcache, (const bf16_t*)vcache, block_table, max_blocks, \
-                tiles, positions, maps, per_kv, kv_heads * maps, kv_heads, dv, page_shift, window, scale, softcap
+                tiles, positions, maps, per_kv, kv_heads * maps, kv_heads, dv, page_shift, window, scale, softcap, partial, per_split, \
+                share, q_slots
 #define AT_DB(N)                                  \
   switch (db) {                                   \
     case 1: rc = launch_tiles<N, 1>(AT_ARGS); break; \
@@ -297,6 +367,7 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
 #undef AT_DB
 #undef AT_ARGS
   if (rc < 0) JLLM_FAIL("attention: cannot reserve LDS");
+  if (partial) attention_dv_merge_kernel<<<dim3(n_rows, q_slots), 64, 0, stream>>>(partial, splits, dv, out, ldo);
   JLLM_CHECK_LAUNCH("attention_dv_bf16");
   return 0;
 }

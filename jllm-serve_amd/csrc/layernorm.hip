@@ -47,30 +47,28 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_seam_kernel(
   const int r = blockIdx.x;
   const size_t src = rows ? (size_t)rows[r] : (size_t)r;
   float* xr = residual + src * d;
-  float x[VPT];
+  // everything the row needs is requested before the first sum: with a few rows a launch is a chain of memory
+  // latencies, and each phase that asked for its own operands added one
+  float x[VPT], t[VPT], wp[VPT], bp[VPT], wn[VPT], bn[VPT], av[VPT];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int i = threadIdx.x + k * LN_THREADS;
-    x[k] = i < d ? xr[i] : 0.f;
+    const bool on = i < d;
+    x[k] = on ? xr[i] : 0.f;
+    t[k] = (on && a) ? ldf(a + (size_t)r * lda, i) : 0.f;
+    av[k] = (on && a2) ? ldf(a2 + (size_t)r * lda2, i) : 0.f;
+    wp[k] = (on && a) ? ldf(w_post, i) : 0.f;
+    bp[k] = (on && a) ? ldf(b_post, i) : 0.f;
+    wn[k] = (on && out) ? ldf(w_next, i) : 0.f;
+    bn[k] = (on && out) ? ldf(b_next, i) : 0.f;
   }
   if (a) {
-    float t[VPT];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      const int i = threadIdx.x + k * LN_THREADS;
-      t[k] = 0.f;
-      if (i < d) {
-        t[k] = s1 * ldf(a + (size_t)r * lda, i);
-        if (a2) t[k] = fmaf(s2, ldf(a2 + (size_t)r * lda2, i), t[k]);
-      }
-    }
+    for (int k = 0; k < VPT; ++k) t[k] = a2 ? fmaf(s2, av[k], s1 * t[k]) : s1 * t[k];
     float mean, rstd;
     ln_stats<VPT>(t, d, red, mean, rstd, eps);
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      const int i = threadIdx.x + k * LN_THREADS;
-      if (i < d) x[k] += (t[k] - mean) * rstd * ldf(w_post, i) + ldf(b_post, i);
-    }
+    for (int k = 0; k < VPT; ++k) x[k] += (t[k] - mean) * rstd * wp[k] + bp[k];
   }
   if (add_vec) {
 #pragma unroll
@@ -92,7 +90,7 @@ __global__ __launch_bounds__(LN_THREADS) void layernorm_seam_kernel(
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       const int i = threadIdx.x + k * LN_THREADS;
-      if (i < d) stf(out + (size_t)r * ldo, i, (x[k] - mean) * rstd * ldf(w_next, i) + ldf(b_next, i));
+      if (i < d) stf(out + (size_t)r * ldo, i, (x[k] - mean) * rstd * wn[k] + bn[k]);
     }
   }
 }
@@ -119,6 +117,8 @@ extern "C" int jllm_layernorm_seam(float* residual, const int* rows, int n, int 
       JLLM_DISPATCH_1(out_dtype, TO, {
         if (d <= LN_THREADS * 4)
           LN_LAUNCH(4);
+        else if (d <= LN_THREADS * 8)
+          LN_LAUNCH(8);
         else if (d <= LN_THREADS * 16)
           LN_LAUNCH(16);
         else

@@ -78,7 +78,7 @@ def _declare(lib) -> None:
         "jllm_layernorm_seam": [_P, _P, _I, _I, _P, _I, _P, _I, _I, _F, _F, _P, _P, _P, _P, _P, _I, _F, _P, _I, _I, _P],
         "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
         "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
-        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _P, _I, _I, _P],
+        "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
         "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
         "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     }
@@ -113,7 +113,7 @@ _OPTIONAL_SIGS = {
     "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_gemm_mfma_grouped_bf16": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _I, _P],
-    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
+    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _I, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -1155,9 +1155,24 @@ def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions
         return False
     n_tiles = int(meta["n_tiles"])
     _i32(tiles, 4 * n_tiles, "tiles")
+    # steps of single rows: the key blocks of a row are shared by as many workgroups as fill the GPU about twice
+    splits, per_split, partial = 1, 0, None
+    T = q.shape[0]
+    if meta.get("single_rows") and n_tiles == T:
+        blocks = -(-max(int(meta.get("max_context", 1)), 1) // 64)
+        want = -(-2 * compute_units() // max(1, n_tiles * kv_heads * maps))  # the heads of a key slot share a workgroup
+        splits = max(1, min(want, blocks // WIDE_SPLIT_MIN_BLOCKS, 64))
+        if splits > 1:
+            per_split = -(-blocks // splits)
+            splits = -(-blocks // per_split)
+            partial = torch.empty((T * heads * maps * splits * (dv + 2),), dtype=torch.float32, device=q.device)
     return _try("jllm_attention_dv_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
                 _ptr(block_table), block_table.shape[1], _ptr(tiles), n_tiles, _ptr(positions), heads, kv_heads, maps, dk, dv,
-                k_cache.shape[2], int(window), float(scale), float(softcap), _stream())
+                k_cache.shape[2], int(window), float(scale), float(softcap), splits, per_split, _ptr(partial),
+                T if meta.get("single_rows") else -1, _stream())
+
+
+WIDE_SPLIT_MIN_BLOCKS = 2  # 64-key blocks a workgroup takes at least when a row's keys are shared out
 
 
 HEAD_GATES = {"sigmoid": 0, "silu": 1}
@@ -1165,10 +1180,12 @@ HEAD_GATES = {"sigmoid": 0, "silu": 1}
 
 def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: torch.dtype, *, lam: float = 0.0,
                  normed: bool = False, eps: float = 0.0, norm_mul: float = 1.0, gain: Optional[torch.Tensor] = None,
-                 gate: Optional[torch.Tensor] = None, gate_fn: str = "sigmoid") -> torch.Tensor:
+                 gate: Optional[torch.Tensor] = None, gate_fn: str = "sigmoid", out: Optional[torch.Tensor] = None,
+                 out_mul: float = 1.0) -> torch.Tensor:
     """From a mixer's heads [T, heads x maps x dv] to the output product's input [T, heads x dv]: with two maps
     o = a1 - lam * a2; ``normed``: o / sqrt(mean(o^2) + eps) * norm_mul per head (times ``gain`` [dv]); with ``gate``
-    ([T, heads x dv], a view with any row stride) times sigmoid(gate) or, ``gate_fn`` "silu", silu(gate)."""
+    ([T, heads x dv], a view with any row stride) times sigmoid(gate) or, ``gate_fn`` "silu", silu(gate); times
+    ``out_mul``. ``out``: where to write (a view with any row stride, [T, heads x dv]) instead of a new tensor."""
     if gate_fn not in HEAD_GATES:
         raise KernelError(f"heads_finish: gate function '{gate_fn}' ({sorted(HEAD_GATES)} are built)")
     _dev(att, gain, gate)
@@ -1182,13 +1199,19 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
             raise KernelError(f"the gate is {tuple(gate.shape)}, expected {(T, heads * dv)}")
     if gain is not None and (gain.numel() != dv or not gain.is_contiguous()):
         raise KernelError(f"the heads' gain must have {dv} entries")
-    out = activation_rows(T, heads * dv, out_dtype, att.device)
+    if out is None:
+        out = activation_rows(T, heads * dv, out_dtype, att.device)
+    else:
+        _dev(out)
+        _rows2d(out, "heads' output")
+        if out.shape != (T, heads * dv):
+            raise KernelError(f"the heads' output is {tuple(out.shape)}, expected {(T, heads * dv)}")
     if T == 0:
         return out
     _call("jllm_heads_finish", _ptr(att), att.stride(0), _code(att.dtype), T, heads, maps, dv, float(lam), 1 if normed else 0,
           float(eps), float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
           gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, HEAD_GATES[gate_fn],
-          _ptr(out), out.stride(0), _code(out.dtype), _stream())
+          float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), _stream())
     return out
 
 

@@ -160,7 +160,8 @@ class SandwichBlock(Part):
         xb = normed_in if isinstance(normed_in, torch.Tensor) else self.norm_in.forward(x)
         then, vec = (next_norm, add_after) if self.ffn is None else (self.norm_post, None)
         scales = getattr(getattr(self.mixer, "spec", None), "scales", ())
-        if hasattr(self.mixer, "outputs") and len(scales) == 2 and hasattr(self.norm_mixer_out, "seam") \
+        if hasattr(self.mixer, "outputs") and not getattr(self.mixer, "fused", False) and len(scales) == 2 \
+                and hasattr(self.norm_mixer_out, "seam") \
                 and (then is None or hasattr(then, "seam")):
             # two weighted branches: their sum is taken inside the seam's launch
             xb = self.norm_mixer_out.seam(x, self.mixer.outputs(xb, step, slot), list(scales), add_vec=vec, then=then)

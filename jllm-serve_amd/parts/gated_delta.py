@@ -78,16 +78,30 @@ class GatedDelta(Part):
         return (StateSpec((s.heads, s.dim, s.vdim), torch.float32),
                 StateSpec((max(s.conv - 1, 1), self.channels), torch.float32))
 
+    def input_projection(self):
+        return self.w_in, None
+
+    def output_weight(self):
+        return self.w_o
+
+    @property
+    def heads_width(self):
+        return self.v_dim
+
     def heads_rows(self, xb, step, slot):
         """The input of the output product, [rows, heads x vdim] in the run's type."""
+        y = ops.gemm(xb, self.w_in, out_dtype=self.build.dtype, exact=self.build.exact)
+        return self.heads_rows_from(y, step, slot)
+
+    def heads_rows_from(self, y, step, slot, out=None, out_mul=1.0):
+        """The same from the input product's result ``y`` (a view with any row stride); ``out``: where to write."""
         s = self.spec
         matrix, tail = slot.state
-        y = ops.gemm(xb, self.w_in, out_dtype=self.build.dtype, exact=self.build.exact)
         qkv = ops.short_conv(y, self.taps, tail, step.row_req, step.state_slots, step.n_requests)
         o = ops.gated_delta(qkv, y, self.a_at, self.b_at, self.a_log, self.dt_bias, matrix, step.row_req, step.state_slots,
                             step.n_requests, s.heads, s.kv_heads, s.dim, s.vdim)
         return ops.heads_finish(o, s.heads, 1, s.vdim, self.build.dtype, normed=True, eps=s.eps, gain=self.gain,
-                                gate=y[:, self.gate_at:self.gate_at + self.v_dim], gate_fn="silu")
+                                gate=y[:, self.gate_at:self.gate_at + self.v_dim], gate_fn="silu", out=out, out_mul=out_mul)
 
     def output(self, xb, step, slot):
         return ops.gemm(self.heads_rows(xb, step, slot), self.w_o, out_dtype=torch.float32, exact=self.build.exact)

@@ -1,10 +1,19 @@
 """Mixers side by side: every branch reads the same input, the result is the sum of the branches' outputs with fixed
 weights. Each branch is a mixer part of its own (any registered kind) with its tensors under a prefix of its own; the
 pages and the state of the layer run are whatever the branches declare (one branch may own pages; the states of all
-branches are handed to them in order)."""
+branches are handed to them in order).
+
+Branches that say what their input and output products are (``input_projection``, ``heads_rows_from``,
+``output_weight``, ``heads_width``) share them: one product with the branches' input weights stacked, each branch
+working from its columns of the result and writing its heads, already multiplied by its weight in the sum, into its
+columns of one buffer, and one output product with the branches' output weights side by side, whose result is the
+weighted sum. A decode layer then has two product launches for the mixer instead of four."""
 from __future__ import annotations
 
+import torch
+
 from ..config.schema import ParallelMixerSpec
+from ..kernels import ops
 from .base import BuildContext, Part, part_factory, register_part
 from .block import sublayer_output
 
@@ -28,6 +37,10 @@ class ParallelMixer(Part):
         if sum(1 for b in self.branches if b.cache_spec() is not None) > 1:
             raise ValueError(f"{prefix}: more than one branch owns pages")
         self.capturable = all(getattr(b, "capturable", True) for b in self.branches)
+        self.build = build
+        self.fused = all(hasattr(b, n) for b in self.branches for n in ("input_projection", "heads_rows_from", "output_weight", "heads_width"))
+        self.w_in = self.b_in = self.w_o = None
+        self._cols = []
         # which of the run's state tensors belong to which branch
         self._state_at = []
         at = 0
@@ -43,6 +56,27 @@ class ParallelMixer(Part):
     def load(self, get):
         for b in self.branches:
             b.load(get)
+        if not self.fused:
+            return
+        ins = [b.input_projection() for b in self.branches]
+        outs = [b.output_weight() for b in self.branches]
+        ws = [w for w, _ in ins]
+        if any(w.dtype != ws[0].dtype for w in ws) or any(o.dtype != outs[0].dtype for o in outs):
+            self.fused = False  # mixed storage types: every branch keeps its own products
+            return
+        self.w_in = torch.cat(ws, dim=0).contiguous()
+        if any(bias is not None for _, bias in ins):
+            self.b_in = torch.cat([bias.to(torch.float32) if bias is not None else torch.zeros(w.shape[0], dtype=torch.float32, device=w.device)
+                                   for w, bias in ins]).contiguous()
+        self.w_o = torch.cat(outs, dim=1).contiguous()
+        at = 0
+        for w, _ in ins:
+            self._cols.append((at, at + w.shape[0]))
+            at += w.shape[0]
+        for b in self.branches:  # the stacked copies are the ones that run
+            for name in ("w_in", "b_in", "w_o"):
+                if hasattr(b, name):
+                    setattr(b, name, None)
 
     def cache_spec(self):
         return next((c for c in (b.cache_spec() for b in self.branches) if c is not None), None)
@@ -67,9 +101,22 @@ class ParallelMixer(Part):
 
     def outputs(self, xb, step, slot):
         """Every branch's output as fp32 rows, in order (an arrangement may weigh and add them itself)."""
+        if self.fused:
+            raise RuntimeError("the branches of this mixer share their products: ask for output()")
         return [sublayer_output(b, xb, step, self._slot(slot, i), self.width) for i, b in enumerate(self.branches)]
 
     def output(self, xb, step, slot):
+        if self.fused:
+            exact = self.build.exact
+            y = ops.gemm(xb, self.w_in, bias=self.b_in, out_dtype=self.build.dtype, exact=exact)
+            heads = ops.activation_rows(step.n_tokens, self.w_o.shape[1], self.build.dtype, y.device)
+            at = 0
+            for i, b in enumerate(self.branches):
+                lo, hi = self._cols[i]
+                b.heads_rows_from(y[:, lo:hi], step, self._slot(slot, i), out=heads[:, at:at + b.heads_width],
+                                  out_mul=self.spec.scales[i])
+                at += b.heads_width
+            return ops.gemm(heads, self.w_o, out_dtype=torch.float32, exact=exact)
         outs = self.outputs(xb, step, slot)
         total = outs[0].mul_(self.spec.scales[0])
         for o, s in zip(outs[1:], self.spec.scales[1:]):

@@ -40,7 +40,8 @@ class WideStepPlanner:
         else:
             runs = [(s.index, s.row0 + r, min(R, s.n - r), s.pos0 + r) for s in batch.segments for r in range(0, s.n, R)]
             runs.sort(key=lambda t: -(t[3] + t[2]))
-        return StepPlan({"tiles": [v for t in runs for v in t]}, {"n_tiles": len(runs)})
+        single = batch.padded or all(s.n == 1 for s in batch.segments)
+        return StepPlan({"tiles": [v for t in runs for v in t]}, {"n_tiles": len(runs), "single_rows": single})
 
 
 class WideAttention(Part):
@@ -125,15 +126,32 @@ class WideAttention(Part):
         if plan is not None:
             tiles = plan.arrays.get("tiles")
             meta["n_tiles"] = plan.facts["n_tiles"]
+            meta["single_rows"] = plan.facts["single_rows"]
             meta["tiles_dev"] = tiles if tiles is not None and tiles.numel() else None
         return meta
 
+    # a mixer that runs beside others on the same input may have its input product and its output product stacked
+    # with theirs (parts/parallel.py): it says what they are, and works from its columns of the stacked result
+    def input_projection(self):
+        return self.w_in, self.b_in
+
+    def output_weight(self):
+        return self.w_o
+
+    @property
+    def heads_width(self):
+        return self.o_dim
+
     def heads_rows(self, xb, step, slot):
         """The input of the output product, [rows, heads x vdim] in the run's type."""
+        y = ops.gemm(xb, self.w_in, bias=self.b_in, out_dtype=self.build.dtype, exact=self.build.exact)
+        return self.heads_rows_from(y, step, slot)
+
+    def heads_rows_from(self, y, step, slot, out=None, out_mul=1.0):
+        """The same from the input product's result ``y`` (a view with any row stride); ``out``: where to write."""
         s, exact = self.spec, self.build.exact
         g = step.groups[slot.group]
         k_cache, v_cache = slot.rows["k"], slot.rows["v"]
-        y = ops.gemm(xb, self.w_in, bias=self.b_in, out_dtype=self.build.dtype, exact=exact)
         cos, sin, rdims = self.rot if self.rot is not None else (None, None, 0)
         ops.qkv_prepare(y, step.positions, g.slots if slot.writes else None, s.heads, s.kv_heads, s.maps, s.dim, s.vdim,
                         k_cache, v_cache, gq=self.g_q, gk=self.g_k, eps=s.eps, cos=cos, sin=sin, rot_dims=rdims,
@@ -145,7 +163,7 @@ class WideAttention(Part):
         gate_at = self.q_dim + self.k_dim + self.v_dim
         gate = y[:, gate_at:gate_at + self.o_dim] if s.out_gate else None
         return ops.heads_finish(att, s.heads, s.maps, s.vdim, self.build.dtype, lam=self.lam, normed=s.maps == 2,
-                                eps=s.eps, norm_mul=1.0 - s.diff, gate=gate)
+                                eps=s.eps, norm_mul=1.0 - s.diff, gate=gate, out=out, out_mul=out_mul)
 
     def output(self, xb, step, slot):
         """The mixer's output as fp32 rows of its own (for arrangements that norm or weigh it before the add)."""

@@ -132,9 +132,17 @@ def test_mixers_alone_through_cache_and_state(name, dtype, built, folders):
         if layer["type"] != "parallel":
             continue
         m = layer["mixer"]
+        from jllm_serve_amd.kernels import ops
         ctx = runner.prepare([StepEntry("side", [0] * T, [])])
         part = model.layers[i].mixer
-        outs = part.outputs(xs[r].to(DEV), ctx, runner.cache.slots[r])
+        assert part.fused, "the two sides share their input and output products"
+        y = ops.gemm(xs[r].to(DEV), part.w_in, bias=part.b_in, out_dtype=act, exact=dtype == "float32")
+        outs, at = [], 0
+        for j, b in enumerate(part.branches):
+            lo, hi = part._cols[j]
+            heads = b.heads_rows_from(y[:, lo:hi], ctx, part._slot(runner.cache.slots[r], j))
+            outs.append(ops.gemm(heads, part.w_o[:, at:at + b.heads_width].contiguous(), out_dtype=torch.float32, exact=dtype == "float32"))
+            at += b.heads_width
         runner.cache.commit("side", T)
         runner.finish("side")
         close(outs[0], P.capped_attention(xs[r].double(), w, f"l{i}.mix.left", m["left"], eps, pos), dtype, f"{name} layer {i} left")
@@ -215,7 +223,7 @@ def test_attention_kernel_on_crafted_keys(dtype, maps, softcap):
         one = ops.attention_dv(q.reshape(T, -1).to(DEV)[sel].contiguous(), kc.to(DEV), vc.to(DEV), bt.repeat(len(rows), 1),
                                torch.arange(len(rows), dtype=torch.int32, device=DEV), pos[sel].contiguous(), H, G, maps, dk, dv,
                                scale, softcap=softcap, out_dtype=torch.float32, exact=exact,
-                               meta={"max_context": T, "requests": len(rows), "rows": len(rows), "n_tiles": len(rows),
+                               meta={"max_context": T, "requests": len(rows), "rows": len(rows), "n_tiles": len(rows), "single_rows": True,
                                      "tiles_dev": torch.tensor([v for i in range(len(rows)) for v in (i, i, 1, -1)],
                                                                dtype=torch.int32, device=DEV)}).cpu()
         assert float((one.view(len(rows), QS, dv).double() - want[rows]).abs().max()) <= tol * float(want.abs().max())

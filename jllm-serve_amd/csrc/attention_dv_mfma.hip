@@ -277,24 +277,25 @@ __global__ __launch_bounds__(256, (DK16 <= 8 && DB <= 4) ? 2 : 1) void attention
     }
 }
 
-// partial [rows][q_slots][splits][dv + 2]: unnormalised sums, then the maximum (as an exponent of two) and the sum
+// partial [rows][q_slots][splits][dv + 2]: unnormalised sums, then the maximum (as an exponent of two) and the sum.
+// Lane z holds split z's maximum and sum (at most 64 splits), so the weights of all splits are known after two wave
+// reductions and the sums' loads are independent of each other.
 __global__ __launch_bounds__(64) void attention_dv_merge_kernel(const float* __restrict__ partial, int splits, int dv,
                                                                 float* __restrict__ out, int ldo) {
   const int t = blockIdx.x, s = blockIdx.y, lane = threadIdx.x;
   const float* pr = partial + ((size_t)t * gridDim.y + s) * splits * (dv + 2);
-  float mx = -INFINITY;
-  for (int z = 0; z < splits; ++z) mx = fmaxf(mx, pr[(size_t)z * (dv + 2) + dv]);
-  float l = 0.f;
-  for (int z = 0; z < splits; ++z) {
-    const float mz = pr[(size_t)z * (dv + 2) + dv];
-    if (mz != -INFINITY) l += pr[(size_t)z * (dv + 2) + dv + 1] * __builtin_amdgcn_exp2f(mz - mx);
-  }
-  const float inv = 1.0f / l;
+  const float mz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv] : -INFINITY;
+  const float lz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
+  const float mx = wave_max(mz);
+  const float wz = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);
+  const float inv = 1.0f / wave_sum(lz * wz);
   for (int d = lane; d < dv; d += 64) {
     float acc = 0.f;
+#pragma unroll 4
     for (int z = 0; z < splits; ++z) {
-      const float mz = pr[(size_t)z * (dv + 2) + dv];
-      if (mz != -INFINITY) acc = fmaf(pr[(size_t)z * (dv + 2) + d], __builtin_amdgcn_exp2f(mz - mx), acc);
+      const float w = __shfl(wz, z, 64);
+      const float v = pr[(size_t)z * (dv + 2) + d];
+      acc = w != 0.f ? fmaf(v, w, acc) : acc;  // a split without keys left its sums unwritten
     }
     out[(size_t)t * ldo + (size_t)s * dv + d] = acc * inv;
   }
@@ -335,7 +336,7 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
   int page_shift = 0;
   while ((1 << page_shift) < page_size) ++page_shift;
   const int q_slots = heads * maps, per_kv = maps * (heads / kv_heads);
-  if (splits > 1 && (!partial || per_split <= 0 || n_rows != n_tiles || splits > 65535)) JLLM_FAIL("attention: %d splits of %d blocks over %d tiles of %d rows", splits, per_split, n_tiles, n_rows);
+  if (splits > 1 && (!partial || per_split <= 0 || n_rows != n_tiles || splits > 64)) JLLM_FAIL("attention: %d splits of %d blocks over %d tiles of %d rows", splits, per_split, n_tiles, n_rows);
   if (splits <= 1) partial = nullptr;
   // tiles of one row: the heads of a key slot share a workgroup (up to the 32 lanes that hold a tile's rows)
   const int share = (n_rows == n_tiles && heads / kv_heads > 1 && heads / kv_heads <= 32) ? heads / kv_heads : 0;

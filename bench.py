@@ -180,11 +180,11 @@ def kebepel_config(z: dict) -> dict:
     """Parallel layers (capped attention with rotation beside a gated delta rule) with a differential attention as
     every second layer's mixer from the second on; every layer has a dense feed-forward."""
     left = {"heads": z["heads"], "kv_heads": z["kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "scale": z["dim"] ** -0.5,
-            "softcap": 50.0, "rot": {"base": 5e5, "dims": z["dim"], "scaling": {"factor": 8.0, "original": 2048, "fast": 32.0, "slow": 1.0}}}
+            "softcap": 30.0, "rot": {"base": 1e6, "dims": z["dim"], "scaling": {"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}
     right = {"heads": z["r_heads"], "kv_heads": z["r_kv_heads"], "dim": z["dim"], "vdim": z["vdim"], "conv": z["conv"]}
-    par = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 0.8, "right_scale": 0.5}, "mlp": {"kind": "dense", "ff": z["ff"]}}
+    par = {"type": "parallel", "mixer": {"left": left, "right": right, "left_scale": 1.0, "right_scale": 1.0}, "mlp": {"kind": "dense", "ff": z["ff"]}}
     att = {"type": "attention", "mixer": {"heads": z["d_heads"], "kv_heads": z["d_kv_heads"], "dim": z["dim"], "vdim": z["d_vdim"],
-                                          "scale": z["dim"] ** -0.5, "diff": 0.3, "q_temp": {"coef": 0.5, "every": 128}},
+                                          "scale": z["dim"] ** -0.5, "diff": 0.2, "q_temp": {"coef": 0.1, "every": 256}},
            "mlp": {"kind": "dense", "ff": z["ff"]}}
     return {"architecture": "Kebepel", "vocab": z["vocab"], "width": z["width"], "norm": {"eps": 1e-6}, "max_positions": 8192,
             "layers": [att if i % 2 else par for i in range(z["layers"])]}

@@ -59,8 +59,8 @@ K_A = {
 K_B = {
     "architecture": "Kebepel", "vocab": 300, "width": 128, "norm": {"eps": 1e-6},
     "layers": [
-        _parallel(_left(8, 4, 64, 32, softcap=20.0, rot_dims=32, base=50000.0, scaling=_yarn(4.0, 32)), _right(4, 4, 64, 32, 4), 0.8, 0.5, 256),
-        _attention(4, 2, 32, 64, 0.3, (0.5, 16), 256),
+        _parallel(_left(8, 2, 64, 48, softcap=20.0, rot_dims=32, base=50000.0, scaling=_yarn(4.0, 32)), _right(4, 4, 64, 32, 4), 0.7, 0.6, 256),
+        _attention(6, 3, 32, 64, 0.35, (0.4, 16), 256),
         _parallel(_left(4, 4, 32, 64, rot_dims=32), _right(4, 2, 32, 64, 4), 1.0, 1.0, 128),
     ],
     "loop": {"start": 0, "stop": 2, "times": 2},

@@ -281,3 +281,81 @@ extern "C" int jllm_heads_finish(const void* att, int lda, int att_dtype, int n_
   JLLM_CHECK_LAUNCH("heads_finish");
   return 0;
 }
+
+// The same finish for heads whose attention was computed in key ranges that are not merged yet: `partial` [rows][heads x
+// maps][splits][dv + 2] holds every range's unnormalised sums, its maximum (as an exponent of two) and its sum, as the
+// matrix-core attention kernel leaves them (attention_dv_mfma.hip). Lane z holds range z's maximum and sum, so the
+// ranges' weights are known after two wave reductions; merging here saves the launch of a merge kernel.
+template <typename TG, typename TW, typename TO>
+__global__ __launch_bounds__(64) void heads_finish_split_kernel(const float* __restrict__ partial, int splits, int maps,
+                                                                int dv, float lambda, int normed, float eps, float norm_mul,
+                                                                const TW* __restrict__ gain, const TG* __restrict__ gate,
+                                                                int ldg, int gate_fn, float out_mul, TO* __restrict__ out,
+                                                                int ldo) {
+  const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+  float o[4] = {0.f, 0.f, 0.f, 0.f};  // dv <= 256
+  for (int m = 0; m < maps; ++m) {
+    const float* pr = partial + (((size_t)t * gridDim.y + h) * maps + m) * splits * (dv + 2);
+    const float mz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv] : -INFINITY;
+    const float lz = lane < splits ? pr[(size_t)lane * (dv + 2) + dv + 1] : 0.f;
+    const float mx = wave_max(mz);
+    const float wz = mz == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mz - mx);
+    const float inv = 1.0f / wave_sum(lz * wz);
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj) {
+      const int j = lane + 64 * jj;
+      if (j >= dv) continue;
+      float acc = 0.f;
+#pragma unroll 4
+      for (int z = 0; z < splits; ++z) {
+        const float w = __shfl(wz, z, 64);
+        const float v = pr[(size_t)z * (dv + 2) + j];
+        acc = w != 0.f ? fmaf(v, w, acc) : acc;  // a range without keys left its sums unwritten
+      }
+      o[jj] = m == 0 ? acc * inv : o[jj] - lambda * (acc * inv);
+    }
+  }
+  float ss = 0.f;
+  if (normed) {
+#pragma unroll
+    for (int jj = 0; jj < 4; ++jj)
+      if (lane + 64 * jj < dv) ss = fmaf(o[jj], o[jj], ss);
+    ss = wave_sum(ss);
+  }
+  const float r = normed ? norm_scale(ss, dv, eps) * norm_mul : 1.0f;
+#pragma unroll
+  for (int jj = 0; jj < 4; ++jj) {
+    const int j = lane + 64 * jj;
+    if (j >= dv) continue;
+    float v = o[jj] * r;
+    if (gain) v *= ldf(gain, j);
+    if (gate) {
+      const float z = ldf(gate + (size_t)t * ldg, (size_t)h * dv + j);
+      v *= (gate_fn == 1 ? z : 1.0f) / (1.0f + expf(-z));
+    }
+    stf(out + (size_t)t * ldo, (size_t)h * dv + j, v * out_mul);
+  }
+}
+
+extern "C" int jllm_heads_finish_split(const float* partial, int splits, int n_tokens, int heads, int maps, int dv, float lambda,
+                                       int normed, float eps, float norm_mul, const void* gain, int gain_dtype, const void* gate,
+                                       int ldg, int gate_dtype, int gate_fn, float out_mul, void* out, int ldo, int out_dtype,
+                                       hipStream_t stream) {
+  if (n_tokens <= 0) return 0;
+  if (heads <= 0 || heads > 65535 || dv <= 0 || dv > 256 || (maps != 1 && maps != 2) || splits < 1 || splits > 64)
+    JLLM_FAIL("heads_finish: %d heads of %d with %d maps in %d key ranges", heads, dv, maps, splits);
+  if (ldo < heads * dv || (gate && ldg < heads * dv)) JLLM_FAIL("heads_finish: short rows");
+  if (gate_fn != 0 && gate_fn != 1) JLLM_FAIL("heads_finish: gate function %d (0 sigmoid and 1 silu are built)", gate_fn);
+  dim3 grid(n_tokens, heads);
+  JLLM_DISPATCH_1(gate_dtype, TG, {
+    JLLM_DISPATCH_1(gain_dtype, TW, {
+      JLLM_DISPATCH_1(out_dtype, TO, {
+        heads_finish_split_kernel<TG, TW, TO><<<grid, 64, 0, stream>>>(partial, splits, maps, dv, lambda, normed, eps, norm_mul,
+                                                                      (const TW*)gain, (const TG*)gate, ldg, gate_fn, out_mul,
+                                                                      (TO*)out, ldo);
+      })
+    })
+  })
+  JLLM_CHECK_LAUNCH("heads_finish_split");
+  return 0;
+}

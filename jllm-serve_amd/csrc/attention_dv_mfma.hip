@@ -321,12 +321,13 @@ static int launch_tiles(dim3 grid, hipStream_t stream, const bf16_t* q, int ldq,
 
 // Returns 1 (declined) for sizes it does not take: dk a multiple of 16 up to 256, dv a multiple of 8 up to 256, bf16.
 // `splits` > 1 (tiles of single rows only): the workgroups of a tile take `per_split` key blocks each and `partial`
-// (fp32, rows x slots x splits x (dv + 2)) carries their results to the merge.
+// (fp32, rows x slots x splits x (dv + 2)) carries their results to the merge (a kernel of its own here, or, with
+// `defer_merge`, the prologue of the kernel that finishes the heads).
 extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ldo, const void* kcache, const void* vcache,
                                       const int* block_table, int max_blocks, const int* tiles, int n_tiles,
                                       const int* positions, int heads, int kv_heads, int maps, int dk, int dv, int page_size,
                                       int window, float scale, float softcap, int splits, int per_split, float* partial,
-                                      int n_rows, hipStream_t stream) {
+                                      int n_rows, int defer_merge, hipStream_t stream) {
   if (n_tiles <= 0) return 0;
   if (heads <= 0 || kv_heads <= 0 || heads % kv_heads != 0 || maps <= 0) JLLM_FAIL("attention: %d query heads over %d kv heads with %d maps", heads, kv_heads, maps);
   if ((dk & 15) || dk < 16 || dk > 256 || (dv & 7) || dv < 8 || dv > 256) return 1;
@@ -368,7 +369,8 @@ extern "C" int jllm_attention_dv_bf16(const void* q, int ldq, float* out, int ld
 #undef AT_DB
 #undef AT_ARGS
   if (rc < 0) JLLM_FAIL("attention: cannot reserve LDS");
-  if (partial) attention_dv_merge_kernel<<<dim3(n_rows, q_slots), 64, 0, stream>>>(partial, splits, dv, out, ldo);
+  // `defer_merge`: the caller's next kernel reads the splits itself (heads_finish_split in attention_dv.hip)
+  if (partial && !defer_merge) attention_dv_merge_kernel<<<dim3(n_rows, q_slots), 64, 0, stream>>>(partial, splits, dv, out, ldo);
   JLLM_CHECK_LAUNCH("attention_dv_bf16");
   return 0;
 }

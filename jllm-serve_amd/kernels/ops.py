@@ -79,6 +79,7 @@ def _declare(lib) -> None:
         "jllm_qkv_prepare": [_P, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _P, _P, _I, _F, _P, _P, _I, _F, _I, _P, _P, _I, _P],
         "jllm_attention_dv_generic": [_P, _I, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _F, _F, _P],
         "jllm_heads_finish": [_P, _I, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
+        "jllm_heads_finish_split": [_P, _I, _I, _I, _I, _I, _F, _I, _F, _F, _P, _I, _P, _I, _I, _I, _F, _P, _I, _I, _P],
         "jllm_short_conv": [_P, _I, _P, _I, _I, _I, _I, _I, _I, _P, _I, _P, _P, _P, _P],
         "jllm_gated_delta": [_P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     }
@@ -113,7 +114,7 @@ _OPTIONAL_SIGS = {
     "jllm_latent_attention_bf16": [_P, _I, _P, _I, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _P],
     "jllm_latent_heads_bf16": [_P, _I, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _I, _I, _P, _P, _P, _P, _I, _P],
     "jllm_gemm_mfma_grouped_bf16": [_P, _I, _P, _P, _P, _I, _I, _I, _I, _I, _I, _F, _P, _I, _I, _P, _I, _P],
-    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _I, _P],
+    "jllm_attention_dv_bf16": [_P, _I, _P, _I, _P, _P, _P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _F, _I, _I, _P, _I, _I, _P],
     "jllm_moe_gemm_bf16": [_P, _I, _I, _P, _P, _I, _P, _I, _I, _I, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _F, _P],
 }
 
@@ -1114,11 +1115,13 @@ def qkv_prepare(qkv: torch.Tensor, positions: torch.Tensor, slots: Optional[torc
 def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, block_table: torch.Tensor,
                  row_req: torch.Tensor, positions: torch.Tensor, heads: int, kv_heads: int, maps: int, dk: int, dv: int,
                  scale: float, *, softcap: float = 0.0, window: int = 0, out_dtype: Optional[torch.dtype] = None,
-                 meta=None, exact: bool = False) -> torch.Tensor:
+                 meta=None, exact: bool = False, defer_merge: bool = False):
     """Causal attention of every row of ``q`` [T, heads x maps x dk] over its request's pages, keys [pages, kv_heads x
     maps, page_size, dk] and values [pages, kv_heads, page_size, dv]: map m of head h reads key slot (h / (heads /
     kv_heads)) * maps + m and value head h / (heads / kv_heads). Scores (q . k) * scale, capped as softcap * tanh(score
-    / softcap) when ``softcap`` > 0. Returns [T, heads x maps x dv] in ``out_dtype`` (default: q's)."""
+    / softcap) when ``softcap`` > 0. Returns [T, heads x maps x dv] in ``out_dtype`` (default: q's). With
+    ``defer_merge`` a step whose rows were computed in key ranges comes back as a ``SplitHeads`` (the ranges' sums,
+    unmerged), which ``heads_finish`` takes in place of the tensor and merges in its prologue."""
     _dev(q, k_cache, v_cache, block_table, row_req, positions)
     _rows2d(q, "q")
     T = q.shape[0]
@@ -1132,9 +1135,11 @@ def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
     out = torch.empty((T, heads * maps * dv), dtype=out_dtype or q.dtype, device=q.device)
     if T == 0:
         return out
-    if not exact and _fast_attention_dv is not None and _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions,
-                                                                        heads, kv_heads, maps, dk, dv, scale, softcap, window, meta):
-        return out
+    if not exact and _fast_attention_dv is not None:
+        got = _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, maps, dk, dv, scale,
+                                 softcap, window, meta, defer_merge)
+        if got is not False:
+            return out if got is True else got
     if not exact:
         _count("general", "jllm_attention_dv_generic")
     _call("jllm_attention_dv_generic", _ptr(q), q.stride(0), _code(q.dtype), _ptr(out), out.stride(0), _code(out.dtype),
@@ -1146,8 +1151,16 @@ def attention_dv(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, 
 WIDE_TILE_ROWS = 128  # rows of one request per tile of the matrix-core kernel (csrc/attention_dv_mfma.hip)
 
 
+class SplitHeads:
+    """Attention rows that were computed in key ranges and are not merged yet: ``partial`` fp32 [rows x (heads x maps) x
+    splits x (dv + 2)] (a range's unnormalised sums, its maximum as an exponent of two, its sum)."""
+
+    def __init__(self, partial: torch.Tensor, splits: int, rows: int, slots: int, dv: int):
+        self.partial, self.splits, self.rows, self.slots, self.dv = partial, splits, rows, slots, dv
+
+
 def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions, heads, kv_heads, maps, dk, dv, scale,
-                       softcap, window, meta) -> bool:
+                       softcap, window, meta, defer_merge=False):
     """The matrix-core kernel: bf16 pages, fp32 out, and the step's rows cut into tiles by the caller (``meta``:
     "tiles_dev" int32 [n_tiles, 4] as (request, first row, rows, first position or -1), "n_tiles")."""
     tiles = meta.get("tiles_dev") if meta else None
@@ -1166,10 +1179,14 @@ def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions
             per_split = -(-blocks // splits)
             splits = -(-blocks // per_split)
             partial = torch.empty((T * heads * maps * splits * (dv + 2),), dtype=torch.float32, device=q.device)
-    return _try("jllm_attention_dv_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
-                _ptr(block_table), block_table.shape[1], _ptr(tiles), n_tiles, _ptr(positions), heads, kv_heads, maps, dk, dv,
-                k_cache.shape[2], int(window), float(scale), float(softcap), splits, per_split, _ptr(partial),
-                T if meta.get("single_rows") else -1, _stream())
+    defer = bool(defer_merge and partial is not None and dv <= 256)
+    ran = _try("jllm_attention_dv_bf16", _ptr(q), q.stride(0), _ptr(out), out.stride(0), _ptr(k_cache), _ptr(v_cache),
+               _ptr(block_table), block_table.shape[1], _ptr(tiles), n_tiles, _ptr(positions), heads, kv_heads, maps, dk, dv,
+               k_cache.shape[2], int(window), float(scale), float(softcap), splits, per_split, _ptr(partial),
+               T if meta.get("single_rows") else -1, 1 if defer else 0, _stream())
+    if ran and defer:
+        return SplitHeads(partial, splits, T, heads * maps, dv)
+    return ran
 
 
 WIDE_SPLIT_MIN_BLOCKS = 2  # 64-key blocks a workgroup takes at least when a row's keys are shared out
@@ -1188,11 +1205,18 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
     ``out_mul``. ``out``: where to write (a view with any row stride, [T, heads x dv]) instead of a new tensor."""
     if gate_fn not in HEAD_GATES:
         raise KernelError(f"heads_finish: gate function '{gate_fn}' ({sorted(HEAD_GATES)} are built)")
-    _dev(att, gain, gate)
-    _rows2d(att, "attention rows")
-    T = att.shape[0]
-    if att.shape[1] != heads * maps * dv:
-        raise KernelError(f"attention rows have {att.shape[1]} entries, expected {heads * maps * dv}")
+    split = att if isinstance(att, SplitHeads) else None
+    if split is not None:
+        if (split.slots, split.dv) != (heads * maps, dv):
+            raise KernelError(f"the unmerged attention has {split.slots} slots of {split.dv}, expected {heads * maps} of {dv}")
+        att, T = split.partial, split.rows
+        _dev(att, gain, gate)
+    else:
+        _dev(att, gain, gate)
+        _rows2d(att, "attention rows")
+        T = att.shape[0]
+        if att.shape[1] != heads * maps * dv:
+            raise KernelError(f"attention rows have {att.shape[1]} entries, expected {heads * maps * dv}")
     if gate is not None:
         _rows2d(gate, "gate")
         if gate.shape != (T, heads * dv):
@@ -1207,6 +1231,12 @@ def heads_finish(att: torch.Tensor, heads: int, maps: int, dv: int, out_dtype: t
         if out.shape != (T, heads * dv):
             raise KernelError(f"the heads' output is {tuple(out.shape)}, expected {(T, heads * dv)}")
     if T == 0:
+        return out
+    if split is not None:
+        _call("jllm_heads_finish_split", _ptr(att), split.splits, T, heads, maps, dv, float(lam), 1 if normed else 0, float(eps),
+              float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),
+              gate.stride(0) if gate is not None else 0, _code(gate.dtype) if gate is not None else F32, HEAD_GATES[gate_fn],
+              float(out_mul), _ptr(out), out.stride(0), _code(out.dtype), _stream())
         return out
     _call("jllm_heads_finish", _ptr(att), att.stride(0), _code(att.dtype), T, heads, maps, dv, float(lam), 1 if normed else 0,
           float(eps), float(norm_mul), _ptr(gain), _code(gain.dtype) if gain is not None else F32, _ptr(gate),

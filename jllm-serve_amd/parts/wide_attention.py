@@ -159,7 +159,7 @@ class WideAttention(Part):
         meta = self._batch_facts(step)
         att = ops.attention_dv(y[:, :self.q_dim], k_cache, v_cache, g.block_table, step.row_req, step.positions, s.heads,
                                s.kv_heads, s.maps, s.dim, s.vdim, s.scale, softcap=s.softcap, window=s.window,
-                               out_dtype=torch.float32, meta=meta, exact=exact)
+                               out_dtype=torch.float32, meta=meta, exact=exact, defer_merge=True)
         gate_at = self.q_dim + self.k_dim + self.v_dim
         gate = y[:, gate_at:gate_at + self.o_dim] if s.out_gate else None
         return ops.heads_finish(att, s.heads, s.maps, s.vdim, self.build.dtype, lam=self.lam, normed=s.maps == 2,

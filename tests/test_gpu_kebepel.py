@@ -227,6 +227,17 @@ def test_attention_kernel_on_crafted_keys(dtype, maps, softcap):
                                      "tiles_dev": torch.tensor([v for i in range(len(rows)) for v in (i, i, 1, -1)],
                                                                dtype=torch.int32, device=DEV)}).cpu()
         assert float((one.view(len(rows), QS, dv).double() - want[rows]).abs().max()) <= tol * float(want.abs().max())
+        if not exact:  # the same rows with the merge of their key ranges left to the kernel that finishes the heads
+            meta = {"max_context": T, "requests": len(rows), "rows": len(rows), "n_tiles": len(rows), "single_rows": True,
+                    "tiles_dev": torch.tensor([v for i in range(len(rows)) for v in (i, i, 1, -1)], dtype=torch.int32, device=DEV)}
+            parts = ops.attention_dv(q.reshape(T, -1).to(DEV)[sel].contiguous(), kc.to(DEV), vc.to(DEV), bt.repeat(len(rows), 1),
+                                     torch.arange(len(rows), dtype=torch.int32, device=DEV), pos[sel].contiguous(), H, G, maps, dk,
+                                     dv, scale, softcap=softcap, out_dtype=torch.float32, meta=meta, defer_merge=True)
+            assert isinstance(parts, ops.SplitHeads) and parts.splits > 1, "the rows' keys were not shared out"
+            kw = dict(lam=0.3, normed=maps == 2, eps=1e-5, norm_mul=0.7)
+            merged_late = ops.heads_finish(parts, H, maps, dv, torch.float32, **kw).cpu()
+            merged_first = ops.heads_finish(one.to(DEV), H, maps, dv, torch.float32, **kw).cpu()
+            assert torch.allclose(merged_late, merged_first, atol=1e-5, rtol=1e-5)
 
 
 def test_qkv_prepare_options():

@@ -80,3 +80,13 @@ class Part:
         ``key`` (equal keys plan once per step) and ``plan(StepBatch) -> StepPlan`` (engine/step.py); the part finds
         the result in ``step.plans[key]``."""
         return []
+
+
+def pad_rows(w: torch.Tensor, multiple: int = 16) -> torch.Tensor:
+    """A stacked weight [N, K] (or bias [N]) with zero rows appended up to a multiple of ``multiple``: the product
+    kernels for few rows take outputs in whole groups of 16, and a stack that ends in a few per-head rows (two numbers
+    per head, say) would otherwise send every product with it to the general kernel. The extra outputs are never read."""
+    extra = -w.shape[0] % multiple
+    if extra == 0:
+        return w
+    return torch.cat([w, torch.zeros((extra,) + tuple(w.shape[1:]), dtype=w.dtype, device=w.device)], dim=0).contiguous()

@@ -23,7 +23,7 @@ from ..cache.manager import StateSpec
 from ..config.schema import GatedDeltaSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import BuildContext, Part, register_part
+from .base import BuildContext, Part, pad_rows, register_part
 
 
 class GatedDelta(Part):
@@ -61,7 +61,7 @@ class GatedDelta(Part):
         nm = self.spec.names
         stack = [get(self._name(n)) for n in ("q", "k", "v", "gate", "decay", "beta")]
         dt = stack[0].dtype if all(t.dtype == stack[0].dtype for t in stack) else torch.float32
-        self.w_in = torch.cat([t.to(dt) for t in stack], dim=0).contiguous()
+        self.w_in = pad_rows(torch.cat([t.to(dt) for t in stack], dim=0).contiguous())
         del stack
         taps = [get(self._name(n, nm.conv_suffix)) for n in "qkv"]
         dt = taps[0].dtype if all(t.dtype == taps[0].dtype for t in taps) else torch.float32

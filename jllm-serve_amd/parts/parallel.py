@@ -14,7 +14,7 @@ import torch
 
 from ..config.schema import ParallelMixerSpec
 from ..kernels import ops
-from .base import BuildContext, Part, part_factory, register_part
+from .base import BuildContext, Part, pad_rows, part_factory, register_part
 from .block import sublayer_output
 
 
@@ -64,10 +64,10 @@ class ParallelMixer(Part):
         if any(w.dtype != ws[0].dtype for w in ws) or any(o.dtype != outs[0].dtype for o in outs):
             self.fused = False  # mixed storage types: every branch keeps its own products
             return
-        self.w_in = torch.cat(ws, dim=0).contiguous()
+        self.w_in = pad_rows(torch.cat(ws, dim=0).contiguous())
         if any(bias is not None for _, bias in ins):
-            self.b_in = torch.cat([bias.to(torch.float32) if bias is not None else torch.zeros(w.shape[0], dtype=torch.float32, device=w.device)
-                                   for w, bias in ins]).contiguous()
+            self.b_in = pad_rows(torch.cat([bias.to(torch.float32) if bias is not None else torch.zeros(w.shape[0], dtype=torch.float32, device=w.device)
+                                            for w, bias in ins]).contiguous())
         self.w_o = torch.cat(outs, dim=1).contiguous()
         at = 0
         for w, _ in ins:

@@ -21,7 +21,7 @@ from ..cache.manager import CacheRow, PageSpec
 from ..config.schema import WideAttentionSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import BuildContext, Part, register_part
+from .base import BuildContext, Part, pad_rows, register_part
 
 
 class WideStepPlanner:
@@ -95,13 +95,13 @@ class WideAttention(Part):
         if s.out_gate:
             stack.append(get(self._name("gate")))
         dt = stack[0].dtype if all(t.dtype == stack[0].dtype for t in stack) else torch.float32
-        self.w_in = torch.cat([t.to(dt) for t in stack], dim=0).contiguous()  # [q | k | v | g] rows
+        self.w_in = pad_rows(torch.cat([t.to(dt) for t in stack], dim=0).contiguous())  # [q | k | v | g] rows
         del stack
         if s.bias:
             b = [get(self._name(n, nm.bias_suffix)).to(torch.float32) for n in "qkv"]
             if s.out_gate:
                 b.append(torch.zeros(self.o_dim, dtype=torch.float32, device=b[0].device))
-            self.b_in = torch.cat(b).contiguous()
+            self.b_in = pad_rows(torch.cat(b).contiguous())
         if s.qk_norm == "whole":
             self.g_q, self.g_k = get(self._name("q", nm.norm_suffix)), get(self._name("k", nm.norm_suffix))
             if self.g_q.dtype != self.g_k.dtype:

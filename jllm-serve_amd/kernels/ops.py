@@ -1173,7 +1173,11 @@ def _fast_attention_dv(q, out, k_cache, v_cache, block_table, row_req, positions
     T = q.shape[0]
     if meta.get("single_rows") and n_tiles == T:
         blocks = -(-max(int(meta.get("max_context", 1)), 1) // 64)
-        want = -(-2 * compute_units() // max(1, n_tiles * kv_heads * maps))  # the heads of a key slot share a workgroup
+        # as many workgroups as are resident at once (two per compute unit; one for the instantiations with keys or
+        # values beyond 128, whose LDS buffers fill a unit): a second round would start its chains of loads all over.
+        # The heads of a key slot share a workgroup
+        resident = (2 if dk <= 128 and dv <= 128 else 1) * compute_units()
+        want = max(1, resident // max(1, n_tiles * kv_heads * maps))
         splits = max(1, min(want, blocks // WIDE_SPLIT_MIN_BLOCKS, 64))
         if splits > 1:
             per_split = -(-blocks // splits)
